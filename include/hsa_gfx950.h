@@ -1,0 +1,135 @@
+/*
+ * hsa_gfx950.h - C ABI of libhsa_gfx950.so: the forward path of hierarchical sparse
+ * attention (sliding window + O(log N) tree neighbours) for AMD MI355X (gfx950).
+ *
+ * Conventions shared by every entry point
+ *   - Plain pointers and sizes only.  Device pointers are borrowed for the call;
+ *     the library allocates nothing and never synchronises: kernels are enqueued
+ *     on `stream` (a hipStream_t passed as void*, NULL = the default stream).
+ *   - Tensors are dense, token-major:  [B, rows, H, D], D fastest.  This is the
+ *     layout of an nn.Linear output viewed as heads, which is what the reference
+ *     kernels consume (hierarchical_attention/modules/attention.py:100-103,182-187).
+ *   - Node index space per batch: rows 0..N-1 are the leaves, row N + ... are the
+ *     tree nodes level by level (level 1 first, root = row 2N-2), the order of
+ *     hierarchical_attention/ops/topology.py:153-169.
+ *   - Return value: 0 on success, a negative errno-style code otherwise; the text
+ *     of the last failure on the calling thread is available from hsa_last_error().
+ *     Nothing throws.  The reference signals misuse with Python `assert`; the
+ *     Python layer above this ABI raises AssertionError for the same conditions.
+ */
+#ifndef HSA_GFX950_H
+#define HSA_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSA_OK 0
+#define HSA_ERR_INVALID (-22)     /* bad shape / pointer / combination of arguments   */
+#define HSA_ERR_UNSUPPORTED (-95) /* valid request this build has no kernel for        */
+#define HSA_ERR_LAUNCH (-5)       /* the HIP runtime rejected the launch               */
+
+/* element types of Q/K/V/Out */
+#define HSA_F32 0
+#define HSA_F16 1
+#define HSA_BF16 2
+
+/* kernel selection for hsa_attn_fwd */
+#define HSA_ATTN_AUTO 0    /* tile kernel when eligible, else the gather kernel */
+#define HSA_ATTN_GATHER 1  /* per-query gather kernel (any dtype, any table)    */
+#define HSA_ATTN_TILE 2    /* MFMA tile kernel or HSA_ERR_UNSUPPORTED           */
+
+int hsa_abi_version(void);
+const char *hsa_last_error(void);
+
+/*
+ * Span attention forward.
+ * Replaces HierarchicalAttentionFunc.forward + hierarchical_attention_forward_kernel
+ * (hierarchical_attention/ops/functional.py:116-168,
+ *  hierarchical_attention/ops/triton/sparse_attn.py:8-179).
+ *
+ *   q, out      [B, N, H, D]
+ *   k, v        [B, M, H, D]   M = 2N-1 in normal use
+ *   idx         device int32 [N, L] neighbour rows (-1 = dead slot), or NULL: use
+ *               the canonical complete-binary-tree table
+ *               idx[n,l] = off_l + ((n >> l) ^ 1), off_0 = 0, off_l = 2N - (N >> (l-1));
+ *               L must then be log2 N and M >= 2N-1
+ *   mask        device bytes [N, L], non-zero = slot masked out.  With idx != NULL:
+ *               NULL means non-causal (the reference's `mask_table is None`), non-NULL
+ *               also masks window keys j > n.  With idx == NULL it must be NULL and
+ *               `causal` selects the canonical mask (bit l of n clear => masked)
+ *   weights     device float [B, N, H, 2R+1+L] softmax weights (window slots first,
+ *               then levels; dead slots 0) or NULL to skip them
+ *   R           window radius: keys n-R..n+R (the reference's `window_size`)
+ *   causal      used only when idx == NULL
+ *   dtype       HSA_F32 / HSA_F16 / HSA_BF16
+ *   algo        HSA_ATTN_*
+ */
+int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
+                 const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
+                 int D, int L, int R, int causal, int dtype, int algo, void *stream);
+
+/* 1 if HSA_ATTN_AUTO would pick the MFMA tile kernel for this problem, else 0. */
+int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype,
+                           int canonical_tables, int want_weights);
+
+/*
+ * One level of the bottom-up parent build.
+ * Replaces BuildParentNodesFunc.forward + build_parent_nodes_forward_kernel
+ * (hierarchical_attention/ops/functional.py:30-63,
+ *  hierarchical_attention/ops/triton/build_parents.py:8-99).
+ *
+ *   qp, kp, vp, out  [B, P, H, D]
+ *   kc, vc           [B, 2P, H, D]    children of parent i are rows 2i, 2i+1
+ *   weights          [B, P, H, 3] in the element type of qp, or NULL
+ *   *_bs             batch strides in elements (0 = dense), so a level can be read
+ *                    from / written into a slice of a larger [B, rows, H, D] buffer
+ */
+int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const void *kc,
+                          const void *vc, void *out, void *weights, int B, int P, int H, int D,
+                          int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
+                          int64_t vc_bs, int64_t out_bs, int dtype, void *stream);
+
+/*
+ * Whole tree in one call: level 1 from the leaves, every further level from the
+ * previous level's output used as both child K and child V (the composition
+ * Out_l = build_parent_nodes(Qp_l, Kp_l, Vp_l, Out_{l-1}, Out_{l-1}) of the op at
+ * hierarchical_attention/ops/functional.py:271-272, i.e. the level loop of
+ * hierarchical_attention/modules/attention.py:119-157 with an identity map
+ * between levels).  Intermediate levels stay on chip.
+ *
+ *   qp, kp, vp  [B, N-1, H, D] level-concatenated (level 1 first, root last)
+ *   k_leaf, v_leaf [B, N, H, D]
+ *   out         [B, N-1, H, D] level-concatenated
+ *   *_bs        batch strides in elements (0 = dense)
+ */
+int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const void *k_leaf,
+                       const void *v_leaf, void *out, int B, int N, int H, int D, int64_t qp_bs,
+                       int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs,
+                       int64_t out_bs, int dtype, void *stream);
+
+/*
+ * Topology tables.  Replaces build_tree_topology
+ * (hierarchical_attention/ops/topology.py:6-150).
+ *   idx [N, L] int32, mask [N, L] bytes (1 = masked), gather [2N-1, 3] int32;
+ *   any of the three may be NULL to skip it.  N must be a power of two.
+ * _host fills host memory on the calling thread; _device enqueues a fill kernel.
+ */
+int hsa_topology_host(int N, int causal, int32_t *idx, uint8_t *mask, int32_t *gather);
+int hsa_topology_device(int N, int causal, int32_t *idx, uint8_t *mask, int32_t *gather,
+                        void *stream);
+
+/*
+ * Initial span nodes: level-by-level pairwise means of x, each level rounded to
+ * the element type.  Replaces generate_span_input_Y
+ * (hierarchical_attention/ops/topology.py:153-169) for power-of-two N.
+ *   x [B, N, C], y [B, N-1, C]
+ */
+int hsa_span_input_y(const void *x, void *y, int B, int N, int C, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSA_GFX950_H */

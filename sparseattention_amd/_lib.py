@@ -1,0 +1,91 @@
+"""ctypes binding of libhsa_gfx950.so (the C ABI declared in include/hsa_gfx950.h).
+
+There is no CPU or PyTorch fallback behind these calls: if the shared library has
+not been built, importing the ops raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_int, c_int64, c_void_p, c_char_p
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhsa_gfx950.so")
+
+HSA_F32, HSA_F16, HSA_BF16 = 0, 1, 2
+ATTN_AUTO, ATTN_GATHER, ATTN_TILE = 0, 1, 2
+_ALGO = {"auto": ATTN_AUTO, "gather": ATTN_GATHER, "tile": ATTN_TILE}
+_DTYPE = {torch.float32: HSA_F32, torch.float16: HSA_F16, torch.bfloat16: HSA_BF16}
+
+_lib = None
+
+
+class HsaError(RuntimeError):
+    pass
+
+
+def _declare(lib):
+    P, I, I64 = c_void_p, c_int, c_int64
+    lib.hsa_abi_version.restype = I
+    lib.hsa_last_error.restype = c_char_p
+    lib.hsa_attn_fwd.argtypes = [P, P, P, P, P, P, P] + [I] * 10 + [P]
+    lib.hsa_attn_fwd.restype = I
+    lib.hsa_attn_fwd_uses_tile.argtypes = [I] * 9
+    lib.hsa_attn_fwd_uses_tile.restype = I
+    lib.hsa_build_parents_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 6 + [I, P]
+    lib.hsa_build_parents_fwd.restype = I
+    lib.hsa_build_tree_fwd.argtypes = [P] * 6 + [I] * 4 + [I64] * 6 + [I, P]
+    lib.hsa_build_tree_fwd.restype = I
+    lib.hsa_topology_host.argtypes = [I, I, P, P, P]
+    lib.hsa_topology_host.restype = I
+    lib.hsa_topology_device.argtypes = [I, I, P, P, P, P]
+    lib.hsa_topology_device.restype = I
+    lib.hsa_span_input_y.argtypes = [P, P, I, I, I, I, P]
+    lib.hsa_span_input_y.restype = I
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HsaError(
+                "libhsa_gfx950.so is missing (%s). Build it first: "
+                "python -m sparseattention_amd._build" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        _declare(handle)
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().hsa_last_error().decode("utf-8", "replace")
+        raise HsaError("%s failed (%d): %s" % (what, rc, msg))
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE[t.dtype]
+    except KeyError:
+        raise AssertionError("unsupported dtype %s (float32, float16, bfloat16 only)" % t.dtype)
+
+
+def algo_code(name: str) -> int:
+    return _ALGO[name]
+
+
+def ptr(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def require_gpu(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise HsaError("this op runs on the GPU only; got a %s tensor" % t.device)
+
+
+def stream_of(t: torch.Tensor):
+    return c_void_p(torch.cuda.current_stream(t.device).cuda_stream)

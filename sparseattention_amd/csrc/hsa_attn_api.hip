@@ -1,0 +1,52 @@
+// hsa_attn_fwd: argument checks and kernel selection for the span attention forward.
+#include "hsa_common.h"
+
+namespace hsa {
+
+int attn_gather_dispatch(const void *q, const void *k, const void *v, const int32_t *idx,
+                         const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
+                         int D, int L, int R, int causal, int dtype, hipStream_t st);
+
+bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
+                        bool want_weights);
+int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
+                       int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st);
+
+}  // namespace hsa
+
+extern "C" {
+
+int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype, int canonical_tables,
+                           int want_weights) {
+    return hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, canonical_tables != 0, want_weights != 0) ? 1 : 0;
+}
+
+int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
+                 const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H, int D,
+                 int L, int R, int causal, int dtype, int algo, void *stream) {
+    HSA_REQUIRE(q && k && v && out, "null pointer");
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
+    HSA_REQUIRE(M >= N, "key rows M=%d < N=%d", M, N);
+    HSA_REQUIRE(L >= 0 && R >= 0, "bad L=%d R=%d", L, R);
+    HSA_REQUIRE(dtype == HSA_F32 || dtype == HSA_F16 || dtype == HSA_BF16, "unknown dtype %d", dtype);
+    const bool canonical = (idx == nullptr);
+    if (canonical) {
+        HSA_REQUIRE(mask == nullptr, "mask must be NULL when idx is NULL (use `causal`)");
+        HSA_REQUIRE(hsa::ilog2_exact(N) == L, "canonical table needs L == log2 N (N=%d L=%d)", N, L);
+        HSA_REQUIRE(M >= 2 * N - 1, "canonical table needs M >= 2N-1 (N=%d M=%d)", N, M);
+    } else {
+        causal = (mask != nullptr);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const bool tile_ok = hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
+    if (algo == HSA_ATTN_TILE && !tile_ok)
+        return hsa::fail(HSA_ERR_UNSUPPORTED,
+                         "tile kernel not available for N=%d H=%d D=%d L=%d R=%d dtype=%d canonical=%d",
+                         N, H, D, L, R, dtype, (int)canonical);
+    if (tile_ok && algo != HSA_ATTN_GATHER)
+        return hsa::attn_tile_dispatch(q, k, v, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0, dtype, st);
+    return hsa::attn_gather_dispatch(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0,
+                                     dtype, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,195 @@
+"""Functional ops: `build_parent_nodes`, `hierarchical_attention` (+ the fused tree build).
+
+Call surface of the reference's hierarchical_attention/ops/functional.py:271-275.
+Each op is a torch.autograd.Function whose forward allocates the output with
+torch and enqueues a kernel of libhsa_gfx950.so on the current stream.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+from . import topology as _topo
+
+
+def _is_canonical(idx_table: torch.Tensor, mask_table: Optional[torch.Tensor], N: int) -> Optional[bool]:
+    """True/False = the tables are the canonical ones for N with that causal flag
+    (known without touching the device); None = unknown table contents."""
+    info = _topo.known_table(idx_table, "idx")
+    if info is None or info[0] != N or idx_table.dtype != torch.int32:
+        return None
+    if mask_table is None:
+        return False
+    minfo = _topo.known_table(mask_table, "mask")
+    if minfo is None or minfo[0] != N or not minfo[1]:
+        return None
+    return True
+
+
+def verify_tables(idx_table: torch.Tensor, mask_table: Optional[torch.Tensor]) -> bool:
+    """Compares tables of unknown origin with the canonical ones on the device (one
+    host sync) and remembers the verdict, so that later calls take the fast path."""
+    N, L = idx_table.shape
+    if N < 1 or (N & (N - 1)) != 0 or L != N.bit_length() - 1:
+        return False
+    canon = _topo.build_tree_topology(N, mask_table is not None, idx_table.device)
+    ok = bool(torch.equal(idx_table.to(torch.int32), canon["forward_idx"]))
+    if ok and mask_table is not None:
+        ok = bool(torch.equal(mask_table.to(torch.bool), canon["forward_mask"]))
+    if ok and idx_table.dtype == torch.int32:
+        _topo._remember(idx_table, "idx", N, mask_table is not None)
+        if mask_table is not None and mask_table.dtype == torch.bool:
+            _topo._remember(mask_table, "mask", N, True)
+    return ok
+
+
+def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16,
+                      return_weights: bool = False, algo: str = "auto"):
+    """Span attention forward on [B,N,H,D] / [B,M,H,D] tensors.
+
+    Returns Out, or (Out, Weights [B,N,H,2R+1+L] fp32) with `return_weights`.
+    `algo`: "auto" | "gather" | "tile".
+    """
+    _lib.require_gpu(Q, K, V, idx_table, mask_table)
+    assert Q.dim() == 4 and K.dim() == 4 and V.dim() == 4, "Q, K, V must be [B, rows, H, D]"
+    assert K.shape == V.shape, "K and V shapes differ"
+    assert Q.dtype == K.dtype == V.dtype, "Q, K, V dtypes differ"
+    B, N, H, D = Q.shape
+    M = K.shape[1]
+    assert K.shape[0] == B and K.shape[2] == H and K.shape[3] == D, "K shape does not match Q"
+    assert idx_table.dim() == 2 and idx_table.shape[0] == N, "idx_table must be [N, levels]"
+    L = idx_table.shape[1]
+    R = int(window_size)
+    assert R >= 0
+    Q, K, V = Q.contiguous(), K.contiguous(), V.contiguous()
+    if mask_table is not None:
+        assert mask_table.shape == idx_table.shape, "mask_table shape mismatch"
+
+    canon = _is_canonical(idx_table, mask_table, N)
+    if canon is None and algo != "gather" and M >= 2 * N - 1:
+        if verify_tables(idx_table, mask_table):
+            canon = mask_table is not None
+    out = torch.empty_like(Q)
+    weights = (torch.empty((B, N, H, 2 * R + 1 + L), device=Q.device, dtype=torch.float32)
+               if return_weights else None)
+    lib = _lib.lib()
+    with torch.cuda.device(Q.device):
+        if canon is not None and M >= 2 * N - 1:
+            rc = lib.hsa_attn_fwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), None, None, _lib.ptr(out),
+                                  _lib.ptr(weights), B, N, M, H, D, L, R, int(canon),
+                                  _lib.dtype_code(Q), _lib.algo_code(algo), _lib.stream_of(Q))
+        else:
+            idx32 = idx_table.to(torch.int32).contiguous()
+            m8 = None
+            if mask_table is not None:
+                m8 = mask_table.contiguous()
+                m8 = m8.view(torch.uint8) if m8.dtype == torch.bool else (m8 != 0).view(torch.uint8)
+            rc = lib.hsa_attn_fwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(idx32), _lib.ptr(m8),
+                                  _lib.ptr(out), _lib.ptr(weights), B, N, M, H, D, L, R, 0,
+                                  _lib.dtype_code(Q), _lib.algo_code(algo), _lib.stream_of(Q))
+    _lib.check(rc, "hsa_attn_fwd")
+    return (out, weights) if return_weights else out
+
+
+def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False):
+    """One level of the parent build on [B,P,H,D] / [B,2P,H,D] tensors."""
+    _lib.require_gpu(Q_p, K_p, V_p, K_c, V_c)
+    Q_p, K_p, V_p, K_c, V_c = (t.contiguous() for t in (Q_p, K_p, V_p, K_c, V_c))
+    B, P, H, D = Q_p.shape
+    assert K_c.shape[1] == 2 * P, "Child count mismatch"
+    assert K_p.shape == Q_p.shape and V_p.shape == Q_p.shape, "parent K/V shape mismatch"
+    assert V_c.shape == K_c.shape and K_c.shape[0] == B and K_c.shape[2:] == Q_p.shape[2:], \
+        "child K/V shape mismatch"
+    assert Q_p.dtype == K_p.dtype == V_p.dtype == K_c.dtype == V_c.dtype, "dtype mismatch"
+    out = torch.empty_like(Q_p)
+    weights = torch.empty((B, P, H, 3), device=Q_p.device, dtype=Q_p.dtype) if return_weights else None
+    with torch.cuda.device(Q_p.device):
+        rc = _lib.lib().hsa_build_parents_fwd(
+            _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
+            _lib.ptr(weights), B, P, H, D, 0, 0, 0, 0, 0, 0, _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
+    _lib.check(rc, "hsa_build_parents_fwd")
+    return (out, weights) if return_weights else out
+
+
+def _batch_stride(t: torch.Tensor) -> int:
+    """Element stride between batches of a [B, rows, H, D] tensor whose rows are dense."""
+    B, rows, H, D = t.shape
+    assert t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D, \
+        "rows of the tensor must be dense [rows, H, D]"
+    return t.stride(0) if B > 1 else rows * H * D
+
+
+def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Every tree level in one call: level 1 from the leaves, level l+1 from level l's
+    outputs used as both child keys and child values.
+
+    Q_p, K_p, V_p [B, N-1, H, D] are level-concatenated (level 1 first, root last) and so
+    is the result.  Tensors may be batch-strided slices of larger buffers (for instance
+    `out = K_full[:, N:]`) as long as each batch's rows are dense.
+    """
+    _lib.require_gpu(Q_p, K_p, V_p, K_leaf, V_leaf, out)
+    B, N, H, D = K_leaf.shape
+    assert N >= 2 and (N & (N - 1)) == 0, "leaf count must be a power of 2"
+    assert Q_p.shape == (B, N - 1, H, D) and K_p.shape == Q_p.shape and V_p.shape == Q_p.shape
+    assert V_leaf.shape == K_leaf.shape
+    if out is None:
+        out = torch.empty((B, N - 1, H, D), dtype=Q_p.dtype, device=Q_p.device)
+    assert out.shape == Q_p.shape and out.dtype == Q_p.dtype
+    ts = [Q_p, K_p, V_p, K_leaf, V_leaf]
+    for i, t in enumerate(ts):
+        if not (t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D):
+            ts[i] = t.contiguous()
+    Q_p, K_p, V_p, K_leaf, V_leaf = ts
+    with torch.cuda.device(Q_p.device):
+        rc = _lib.lib().hsa_build_tree_fwd(
+            _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_leaf), _lib.ptr(V_leaf), _lib.ptr(out),
+            B, N, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
+            _batch_stride(K_leaf), _batch_stride(V_leaf), _batch_stride(out), _lib.dtype_code(Q_p),
+            _lib.stream_of(Q_p))
+    _lib.check(rc, "hsa_build_tree_fwd")
+    return out
+
+
+class BuildParentNodesFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, Q_p, K_p, V_p, K_c, V_c):
+        need_grad = any(ctx.needs_input_grad)
+        if need_grad:
+            out, w = build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights=True)
+            ctx.save_for_backward(Q_p, K_p, V_p, K_c, V_c, w)
+            return out
+        return build_parents_forward(Q_p, K_p, V_p, K_c, V_c)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("build_parent_nodes: this build provides the forward pass only")
+
+
+class HierarchicalAttentionFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, Q, K, V, idx_table, gather_table, mask_table=None, window_size=16):
+        need_grad = any(ctx.needs_input_grad[:3])
+        if need_grad:
+            out, w = attention_forward(Q, K, V, idx_table, mask_table, window_size, return_weights=True)
+            ctx.save_for_backward(Q, K, V, idx_table, gather_table, w, mask_table)
+            ctx.window_size = int(window_size)
+            return out
+        return attention_forward(Q, K, V, idx_table, mask_table, window_size)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        raise NotImplementedError("hierarchical_attention: this build provides the forward pass only")
+
+
+def build_parent_nodes(Q_p, K_p, V_p, K_c, V_c):
+    """Parent i attends over {itself, children 2i and 2i+1}; returns [B, P, H, D]."""
+    return BuildParentNodesFunc.apply(Q_p, K_p, V_p, K_c, V_c)
+
+
+def hierarchical_attention(Q, K, V, idx_table, gather_table, mask_table=None, window_size=16):
+    """Each leaf query attends to keys n-R..n+R plus one tree node per level.
+    `mask_table is None` selects the non-causal mode; `gather_table` is unused by the
+    forward pass."""
+    return HierarchicalAttentionFunc.apply(Q, K, V, idx_table, gather_table, mask_table, window_size)
