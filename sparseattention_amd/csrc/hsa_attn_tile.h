@@ -1,0 +1,366 @@
+// Span attention forward, MFMA tile kernel (16-bit element types, canonical tree tables).
+//
+// Work decomposition
+//   A wavefront owns one (batch, head) and a strip of consecutive blocks of 16 queries.
+//   For a 16-query block starting at q0 (a multiple of 16) the keys every query of the
+//   block can attend to are
+//     - the leaf blocks q0-16*NBW .. q0 (.. q0+16*NBW when not causal), NBW = ceil(R/16);
+//       the level-0 neighbour n^1 lies inside the block's own leaf block;
+//     - the 14 tree nodes of levels 1..3 under the block's level-4 ancestor
+//       (8 + 4 + 2 consecutive rows) and one sibling node per level 4..L-1, which is the
+//       same for all 16 queries: 14 + (L-4) <= 32 "tree slots" = two more key blocks.
+//   So the block's scores are a handful of dense 16x16 tiles with a per-element
+//   multiplicity mask (0: not attended, 1, or 2 for the leaf n^1 that is both a window
+//   key and the level-0 neighbour).
+//
+// Data flow (no LDS): every operand is loaded from global memory directly in MFMA
+// operand layout, 16 bytes per lane (lane = row, four lane groups = four 8-element
+// pieces of 32 channels).
+//     S^T[key, query] = K_blk . Q_blk^T            v_mfma_f32_16x16x32 (A = K rows, B = Q rows)
+//     V^T-operand     = V_blk . Pi                 the same MFMA with a 0/1 selection matrix
+//                                                  moves V into "lane = channel, regs = keys"
+//     O^T[ch, query]  = V^T . P^T                  v_mfma_f32_16x16x16 (A, B both come from
+//                                                  MFMA results, whose layouts agree)
+// The selection matrix orders channels so that a lane ends up holding 8 consecutive
+// output channels of one query: the result is stored with one 16-byte store per 32
+// channels, in the same addressing pattern as the Q loads.
+// Leaf K / transposed-V operands slide along the strip in registers, so inside a strip
+// every K/V row is fetched once; the next block's operands are requested before the
+// current block is computed.
+#pragma once
+
+#include "hsa_common.h"
+
+namespace hsa {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mma;
+
+template <> struct Mma<BF16> {
+    static constexpr uint16_t kOne = 0x3f80;
+    static __device__ __forceinline__ f32x4 k32(uint4 a, uint4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 k16(uint2 a, uint2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
+                                                         __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+    }
+    // round-to-nearest-even pair
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+    }
+    // the inputs are exactly representable: keep the high halves
+    static __device__ __forceinline__ uint32_t pack_exact(float a, float b) {
+        return (__float_as_uint(a) >> 16) | (__float_as_uint(b) & 0xffff0000u);
+    }
+};
+
+template <> struct Mma<F16> {
+    static constexpr uint16_t kOne = 0x3c00;
+    static __device__ __forceinline__ f32x4 k32(uint4 a, uint4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 k16(uint2 a, uint2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
+                                                     __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+    }
+    static __device__ __forceinline__ uint32_t pack_exact(float a, float b) { return pack(a, b); }
+};
+
+constexpr int TILE_Q = 16;           // queries per block
+constexpr int TILE_TREE_BLOCKS = 2;  // 32 tree slots
+constexpr int TILE_MAX_LEVELS = 22;  // 14 + (L - 4) <= 32
+constexpr float NEG_INF = -__builtin_inff();
+
+struct TileParams {
+    const uint16_t *q, *k, *v;
+    uint16_t *out;
+    int B, N, M, H, L, R;
+    int SB;       // query blocks per strip
+    int NS;       // strips per sequence
+    int n_units;  // B * NS * H
+    float scale_log2e;
+};
+
+// wavefronts per workgroup: 8 (two per SIMD, <= 256 VGPRs each) up to 64 channels,
+// 4 (one per SIMD, <= 512 VGPRs) for 128 channels
+template <int D> constexpr int tile_max_wpb() { return D > 64 ? 4 : 8; }
+
+template <typename T, int D, int NBW, bool CAUSAL>
+__global__ void __launch_bounds__(tile_max_wpb<D>() * 64)
+attn_tile_kernel(TileParams p) {
+    using M_ = Mma<T>;
+    constexpr int KS = D / 32;                         // 32-channel steps of the QK contraction
+    constexpr int NJ = D / 16;                         // 16-channel output tiles
+    constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // leaf key blocks per query block
+    constexpr int NEWC = NKL - 1;                      // the leaf block that enters each step
+
+    const int lane = threadIdx.x & 63;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int wpb = blockDim.x >> 6;
+
+    // workgroups that are consecutive in `logical` run on the same XCD (hardware hands
+    // consecutive workgroup ids to the 8 XCDs in turn), so strips that share halo rows
+    // and upper tree nodes share an L2.
+    int wg = blockIdx.x;
+    const int nwg = gridDim.x;
+    if ((nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);
+    const int unit = wg * wpb + (threadIdx.x >> 6);
+    if (unit >= p.n_units) return;
+    const int h = unit % p.H;
+    const int s = (unit / p.H) % p.NS;
+    const int b = unit / (p.H * p.NS);
+
+    const int N = p.N, L = p.L, R = p.R;
+    const int NB = N / TILE_Q;
+    const int blk0 = s * p.SB;
+    const int nblk = (NB - blk0) < p.SB ? (NB - blk0) : p.SB;
+    const size_t rs = (size_t)p.H * D;  // elements between consecutive rows
+    const uint16_t *Qb = p.q + ((size_t)b * N * p.H + h) * D + 8 * g;
+    const uint16_t *Kb = p.k + ((size_t)b * p.M * p.H + h) * D + 8 * g;
+    const uint16_t *Vb = p.v + ((size_t)b * p.M * p.H + h) * D + 8 * g;
+    uint16_t *Ob = p.out + ((size_t)b * N * p.H + h) * D + 8 * g;
+
+    // ---- lane constants -------------------------------------------------------------
+    // selection matrices: output column n of tile jj picks channel 8*(n/4) + 4*jj + n%4
+    // of the 32-channel step; as a B operand this lane (column r16, rows 8g..8g+7) holds
+    // a single one when g == r16/4.
+    uint4 Pi[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+        uint32_t w[4] = {0, 0, 0, 0};
+        if (g == (r16 >> 2)) {
+            const int e = 4 * jj + (r16 & 3);  // element 0..7 inside this lane's 8 rows
+            w[e >> 1] = (uint32_t)M_::kOne << (16 * (e & 1));
+        }
+        Pi[jj] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+
+    // additive score bias of the leaf blocks (log2 of the multiplicity, -inf = not attended)
+    float biasL[NKL][4];
+#pragma unroll
+    for (int c = 0; c < NKL; ++c) {
+        const int dlt = TILE_Q * (c - NBW);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kl = 4 * g + i;
+            const int diff = dlt + kl - r16;
+            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+            const bool sib = dlt == 0 && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
+            const int cnt = (int)win + (int)sib;
+            biasL[c][i] = cnt == 0 ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+        }
+    }
+
+    // tree slots: slot s in [0,32).  0..7 level 1, 8..11 level 2, 12..13 level 3,
+    // 14+u level 4+u.  (a) the slot whose row this lane loads, per tree block;
+    // (b) level and liveness of the slots whose scores this lane holds.
+    int ld_off[TILE_TREE_BLOCKS], ld_lvl[TILE_TREE_BLOCKS], ld_add[TILE_TREE_BLOCKS], ld_xor[TILE_TREE_BLOCKS];
+#pragma unroll
+    for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
+        const int sl = 16 * t + r16;
+        int lvl, add, x;
+        if (sl < 8) { lvl = 1; add = sl; x = 0; }
+        else if (sl < 12) { lvl = 2; add = sl - 8; x = 0; }
+        else if (sl < 14) { lvl = 3; add = sl - 12; x = 0; }
+        else { lvl = 4 + (sl - 14); add = 0; x = 1; }
+        if (lvl >= L) { lvl = 1; add = 0; x = 0; }  // unused slot: point at a valid row
+        ld_lvl[t] = lvl; ld_add[t] = add; ld_xor[t] = x;
+        ld_off[t] = level_offset(N, lvl);
+    }
+    float biasT[TILE_TREE_BLOCKS][4];   // constant part
+    int upT[TILE_TREE_BLOCKS][4];       // level of an upper slot (>= 4), or -1
+#pragma unroll
+    for (int t = 0; t < TILE_TREE_BLOCKS; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int sl = 16 * t + 4 * g + i;
+            int lvl, pl;
+            if (sl < 8) { lvl = 1; pl = sl; }
+            else if (sl < 12) { lvl = 2; pl = sl - 8; }
+            else if (sl < 14) { lvl = 3; pl = sl - 12; }
+            else { lvl = 4 + (sl - 14); pl = -1; }
+            bool live;
+            upT[t][i] = -1;
+            if (pl >= 0) {
+                live = pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1));
+            } else {
+                live = lvl < L;
+                if (CAUSAL && live) upT[t][i] = lvl;
+            }
+            biasT[t][i] = live ? 0.0f : NEG_INF;
+        }
+
+    // ---- loaders ----------------------------------------------------------------------
+    auto load_rows = [&](const uint16_t *base, int row, uint4 (&dst)[KS]) {
+        const uint16_t *ptr = base + (size_t)row * rs;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const uint4 *>(ptr + 32 * ks);
+    };
+    auto leaf_row = [&](int kb) {  // first row of leaf block kb, clamped into the sequence
+        kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
+        return kb * TILE_Q + r16;
+    };
+    auto tree_row = [&](int t, int q0) {
+        return ld_off[t] + ((((q0 >> ld_lvl[t]) + ld_add[t])) ^ ld_xor[t]);
+    };
+    auto transpose_v = [&](const uint4 (&raw)[KS], uint2 (&dst)[NJ]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            f32x4 r = M_::k32(raw[j >> 1], Pi[j & 1], z);
+            dst[j] = make_uint2(M_::pack_exact(r[0], r[1]), M_::pack_exact(r[2], r[3]));
+        }
+    };
+
+    // ---- rolling leaf operands ----------------------------------------------------------
+    uint4 Kl[NKL][KS];
+    uint2 Vl[NKL][NJ];
+#pragma unroll
+    for (int c = 0; c < NKL - 1; ++c) {
+        const int row = leaf_row(blk0 - NBW + c);
+        uint4 raw[KS];
+        load_rows(Kb, row, Kl[c]);
+        load_rows(Vb, row, raw);
+        transpose_v(raw, Vl[c]);
+    }
+
+    // operands requested one block ahead
+    uint4 nQ[KS], nK[KS], nV[KS], nKt[TILE_TREE_BLOCKS][KS], nVt[TILE_TREE_BLOCKS][KS];
+    auto request = [&](int blk) {
+        const int q0 = blk * TILE_Q;
+        load_rows(Qb, q0 + r16, nQ);
+        const int row = leaf_row(blk + (CAUSAL ? 0 : NBW));
+        load_rows(Kb, row, nK);
+        load_rows(Vb, row, nV);
+#pragma unroll
+        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
+            const int tr = tree_row(t, q0);
+            load_rows(Kb, tr, nKt[t]);
+            load_rows(Vb, tr, nVt[t]);
+        }
+    };
+    request(blk0);
+
+    for (int it = 0; it < nblk; ++it) {
+        const int blk = blk0 + it;
+        const int q0 = blk * TILE_Q;
+        uint4 Qf[KS], Kt[TILE_TREE_BLOCKS][KS], rawV[KS], rawVt[TILE_TREE_BLOCKS][KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            Qf[ks] = nQ[ks];
+            Kl[NEWC][ks] = nK[ks];
+            rawV[ks] = nV[ks];
+#pragma unroll
+            for (int t = 0; t < TILE_TREE_BLOCKS; ++t) { Kt[t][ks] = nKt[t][ks]; rawVt[t][ks] = nVt[t][ks]; }
+        }
+        if (it + 1 < nblk) request(blk + 1);
+
+        // scores, transposed: S[c][i] = score(key 4g+i of block c, query r16)
+        float sc[NKL + TILE_TREE_BLOCKS][4];
+        float mx = NEG_INF;
+#pragma unroll
+        for (int c = 0; c < NKL; ++c) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) acc = M_::k32(Kl[c][ks], Qf[ks], acc);
+            const int kb = blk - NBW + c;
+            const bool inside = kb >= 0 && kb < NB;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float v = inside ? fmaf(acc[i], p.scale_log2e, biasL[c][i]) : NEG_INF;
+                sc[c][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) acc = M_::k32(Kt[t][ks], Qf[ks], acc);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float bias = biasT[t][i];
+                if (CAUSAL) {
+                    const int lv = upT[t][i];
+                    if (lv >= 0 && ((q0 >> lv) & 1) == 0) bias = NEG_INF;
+                }
+                float v = fmaf(acc[i], p.scale_log2e, bias);
+                sc[NKL + t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+
+        // new value blocks into "lane = channel, regs = keys" form
+        uint2 Vt[TILE_TREE_BLOCKS][NJ];
+        transpose_v(rawV, Vl[NEWC]);
+#pragma unroll
+        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) transpose_v(rawVt[t], Vt[t]);
+
+        float den = 0.f;
+        uint2 P[NKL + TILE_TREE_BLOCKS];
+#pragma unroll
+        for (int c = 0; c < NKL + TILE_TREE_BLOCKS; ++c) {
+            float e[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                e[i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
+                den += e[i];
+            }
+            P[c] = make_uint2(M_::pack(e[0], e[1]), M_::pack(e[2], e[3]));
+        }
+        den += __shfl_xor(den, 16, 64);
+        den += __shfl_xor(den, 32, 64);
+        const float inv = 1.0f / den;
+
+        uint16_t *optr = Ob + (size_t)(q0 + r16) * rs;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            uint32_t w[4];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+                const int j = 2 * ks + jj;
+                f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NKL; ++c) o = M_::k16(Vl[c][j], P[c], o);
+#pragma unroll
+                for (int t = 0; t < TILE_TREE_BLOCKS; ++t) o = M_::k16(Vt[t][j], P[NKL + t], o);
+                w[2 * jj] = M_::pack(o[0] * inv, o[1] * inv);
+                w[2 * jj + 1] = M_::pack(o[2] * inv, o[3] * inv);
+            }
+            *reinterpret_cast<uint4 *>(optr + 32 * ks) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+
+        // slide the leaf window by one block
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) Kl[c][ks] = Kl[c + 1][ks];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) Vl[c][j] = Vl[c + 1][j];
+        }
+    }
+}
+
+template <typename T, int D>
+int attn_tile_launch_td(const TileParams &p, int nbw, bool causal, int wpb, hipStream_t st);
+
+}  // namespace hsa

@@ -1,9 +1,57 @@
-// placeholder: tile kernel not built yet
-#include "hsa_common.h"
+// Eligibility test and launch parameters of the MFMA tile kernel.
+#include "hsa_attn_tile.h"
+
+#include <stdlib.h>
+
 namespace hsa {
-bool attn_tile_eligible(int, int, int, int, int, int, int, bool, bool) { return false; }
-int attn_tile_dispatch(const void *, const void *, const void *, void *, float *, int, int, int, int, int,
-                       int, int, int, int, hipStream_t) {
-    return fail(HSA_ERR_UNSUPPORTED, "tile kernel not built");
+
+constexpr int TILE_MAX_NBW = 2;
+
+bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
+                        bool want_weights) {
+    (void)H;
+    if (!canonical || want_weights) return false;
+    if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
+    if (D != 64 && D != 128) return false;
+    if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS) return false;
+    if (M < 2 * N - 1) return false;
+    if ((R + TILE_Q - 1) / TILE_Q > TILE_MAX_NBW) return false;
+    return true;
 }
+
+int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
+                       int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st) {
+    (void)weights;
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fail(HSA_ERR_INVALID, "tile kernel needs 16-byte aligned tensors");
+    TileParams p;
+    p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v;
+    p.out = (uint16_t *)out;
+    p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
+    const int NB = N / TILE_Q;
+    // strip length: long enough to amortise the halo and to prefetch, short enough to give
+    // every SIMD of the 256 CUs at least two wavefronts
+    const long block_units = (long)B * H * NB;
+    int sb = (int)(block_units / 2048);
+    if (sb < 1) sb = 1;
+    if (sb > 8) sb = 8;
+    if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x >= 1) sb = x; }
+    if (sb > NB) sb = NB;
+    p.SB = sb;
+    p.NS = (NB + sb - 1) / sb;
+    const long units = (long)B * p.NS * H;
+    if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.n_units = (int)units;
+    p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
+    int wpb = 8;
+    if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
+    const int nbw = (R + TILE_Q - 1) / TILE_Q;
+    if (dtype == HSA_BF16) {
+        if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, wpb, st);
+        return attn_tile_launch_td<BF16, 128>(p, nbw, causal != 0, wpb, st);
+    }
+    if (D == 64) return attn_tile_launch_td<F16, 64>(p, nbw, causal != 0, wpb, st);
+    return attn_tile_launch_td<F16, 128>(p, nbw, causal != 0, wpb, st);
+}
+
 }  // namespace hsa

@@ -228,3 +228,75 @@ def test_cfg2_gather_full_size(causal, bf):
     out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
                                t["forward_mask"] if causal else None, R, algo="gather")
     _bf_check(bf, q, k, v, N, R, causal, out, torch.bfloat16)
+
+
+# ---------------------------------------------------------------- span attention, MFMA tile kernel
+TILE_CASES = [  # B, N, H, D, R
+    (2, 16, 2, 64, 1),
+    (1, 32, 3, 64, 16),
+    (2, 64, 8, 64, 8),
+    (2, 256, 4, 64, 16),
+    (1, 512, 12, 64, 20),
+    (1, 128, 2, 128, 32),
+    (2, 64, 2, 128, 5),
+    (1, 64, 2, 64, 0),
+]
+
+
+@pytest.mark.parametrize("case", TILE_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("strip", [None, "1", "3"])
+def test_attention_tile_vs_oracle(case, dtype, causal, strip, monkeypatch):
+    B, N, H, D, R = case
+    if strip is not None:
+        monkeypatch.setenv("HSA_ATTN_TILE_SB", strip)
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    o = oracle.topology_tables(N, causal)
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                               t["forward_mask"] if causal else None, R, algo="tile")
+    want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
+                                compute_dtype=torch.float64)
+    assert_close(out, want, dtype, "tile")
+
+
+def test_tile_is_the_default_for_the_headline_shape():
+    from sparseattention_amd import _lib
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 1, 0) == 1
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_F32, 1, 0) == 0
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 0, 0) == 0
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_cfg2_tile_full_size(causal, bf):
+    B, H, N, D, R = 16, 8, 512, 64, 8
+    q, k, v = make_qkv(B, N, H, D, torch.bfloat16, seed=0, scale=1.0 / 8)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    out = sa.hierarchical_attention(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], t["backward_gather"],
+                                    t["forward_mask"] if causal else None, R)
+    _bf_check(bf, q, k, v, N, R, causal, out, torch.bfloat16)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_cfg3_headline_full_size(causal, bf):
+    """B8 H8 N2048 d64 bf16 R16 with the parents built by the tree kernel."""
+    B, H, N, D, R = 8, 8, 2048, 64, 16
+    g = torch.Generator().manual_seed(0)
+    mk = lambda rows: torch.randn(B, rows, H, D, generator=g).to(torch.bfloat16)
+    q, kl, vl, qp, kp, vp = mk(N), mk(N), mk(N), mk(N - 1), mk(N - 1), mk(N - 1)
+    kfull = torch.empty(B, 2 * N - 1, H, D, dtype=torch.bfloat16, device=DEV)
+    vfull = torch.empty_like(kfull)
+    kfull[:, :N] = kl.to(DEV)
+    vfull[:, :N] = vl.to(DEV)
+    sa.build_tree(qp.to(DEV), kp.to(DEV), vp.to(DEV), kfull[:, :N], vfull[:, :N], out=kfull[:, N:])
+    vfull[:, N:] = kfull[:, N:]
+    tree = oracle.build_tree_ref(qp, kp, vp, kl, vl, compute_dtype=torch.float64)
+    assert_close(kfull[:, N:], tree, torch.bfloat16, "tree")
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    out = sa.hierarchical_attention(q.to(DEV), kfull, vfull, t["forward_idx"], t["backward_gather"],
+                                    t["forward_mask"] if causal else None, R)
+    _bf_check(bf, q, kfull.cpu(), vfull.cpu(), N, R, causal, out, torch.bfloat16)
+    out_g = fn.attention_forward(q.to(DEV), kfull, vfull, t["forward_idx"],
+                                 t["forward_mask"] if causal else None, R, algo="gather")
+    assert (out.float() - out_g.float()).abs().max() < 2e-2
