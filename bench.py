@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the hierarchical sparse attention forward path on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input resident in HBM:
+the bottom-up tree build (every BuildParentNodes level) that produces the node rows of
+K_full / V_full, followed by the span attention forward.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg5]
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: (B, H, N, D, R, input scale, description)
+    "cfg2": (16, 8, 512, 64, 8, 1.0 / 8, "B16 H8 N512 d64 bf16 SWA8 causal"),
+    "cfg3": (8, 8, 2048, 64, 16, 1.0, "B8 H8 N2048 d64 bf16 SWA16 causal, parents built by the tree kernel"),
+    "cfg5": (1, 16, 65536, 128, 32, 1.0, "B1 H16 N65536 d128 bf16 SWA32 causal"),
+}
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--noncausal", action="store_true")
+    ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    return ap.parse_args()
+
+
+def cpu_baseline(B, H, N, D, R, causal, scale, budget_s):
+    """Times the CPU restatement of the reference's PyTorch algorithm (tree build level by
+    level + gather/einsum span attention) on this host's cores, bf16 tensors like the GPU run."""
+    import torch
+    import oracle
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else int(os.environ["OMP_NUM_THREADS"])
+    torch.set_num_threads(cores)
+    g = torch.Generator().manual_seed(0)
+    bs = min(B, 2)   # bounded sample: a slice of the batch, same N/H/D/R
+    mk = lambda rows: (torch.randn(bs, rows, H, D, generator=g) * scale).to(torch.bfloat16)
+    q, kl, vl, qp, kp, vp = mk(N), mk(N), mk(N), mk(N - 1), mk(N - 1), mk(N - 1)
+    t = oracle.topology_tables(N, causal)
+    m = t["forward_mask"] if causal else None
+
+    def one():
+        tree = oracle.build_tree_ref(qp, kp, vp, kl, vl)
+        kf = torch.cat([kl, tree], 1)
+        vf = torch.cat([vl, tree], 1)
+        return oracle.attention_ref(q, kf, vf, t["forward_idx"], m, R)
+
+    one()
+    times, t_end = [], time.perf_counter() + budget_s
+    while len(times) < 3 or (time.perf_counter() < t_end and len(times) < 50):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": bs * N * H / med, "unit": "head-queries/s", "cores": cores, "kind": "port",
+            "sample": "%d of %d batches of the same workload (bf16, torch CPU, %d threads), median of %d passes"
+                      % (bs, B, cores, len(times))}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this build has no multi-GPU path (every (batch, head) "
+              "is independent; see DESIGN.md for how it would shard). Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from sparseattention_amd import _lib
+    import sparseattention_amd as sa
+
+    B, H, N, D, R, scale, desc = WORKLOADS[args.workload]
+    causal = not args.noncausal
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.lib()
+    L = N.bit_length() - 1
+    M = 2 * N - 1
+    e = 2
+    set_bytes = e * B * H * D * (N + 2 * M + N + 3 * (N - 1))
+    nsets = args.sets or max(3, -(-512 * 2**20 // set_bytes))
+
+    g = torch.Generator().manual_seed(0)
+    sets = []
+    for _ in range(nsets):
+        mk = lambda rows: (torch.randn(B, rows, H, D, generator=g) * scale).to(torch.bfloat16).to(dev)
+        s = {"q": mk(N), "qp": mk(N - 1), "kp": mk(N - 1), "vp": mk(N - 1),
+             "kfull": torch.empty(B, M, H, D, dtype=torch.bfloat16, device=dev),
+             "vfull": torch.empty(B, M, H, D, dtype=torch.bfloat16, device=dev),
+             "out": torch.empty(B, N, H, D, dtype=torch.bfloat16, device=dev)}
+        s["kfull"][:, :N] = mk(N)
+        s["vfull"][:, :N] = mk(N)
+        sets.append(s)
+
+    stream = torch.cuda.current_stream(dev)
+    st = ctypes.c_void_p(stream.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    node_off = N * H * D * e
+    full_bs = M * H * D
+
+    def tree_args(s):
+        return (P(s["qp"]), P(s["kp"]), P(s["vp"]), P(s["kfull"]), P(s["vfull"]),
+                ctypes.c_void_p(s["kfull"].data_ptr() + node_off), ctypes.c_void_p(s["vfull"].data_ptr() + node_off),
+                B, N, H, D, 0, 0, 0, full_bs, full_bs, full_bs, full_bs, _lib.HSA_BF16, st)
+
+    def attn_args(s):
+        return (P(s["q"]), P(s["kfull"]), P(s["vfull"]), None, None, P(s["out"]), None,
+                B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st)
+
+    targs = [tree_args(s) for s in sets]
+    aargs = [attn_args(s) for s in sets]
+    assert lib.hsa_attn_fwd_uses_tile(N, M, H, D, L, R, _lib.HSA_BF16, 1, 0) == 1
+
+    def step(i):
+        rc = lib.hsa_build_tree_fwd(*targs[i % nsets])
+        rc |= lib.hsa_attn_fwd(*aargs[i % nsets])
+        return rc
+
+    for i in range(args.warmup):
+        assert step(i) == 0, lib.hsa_last_error()
+    torch.cuda.synchronize()
+
+    # --- timed region: exactly K steps, events around every attention launch -------------
+    K = args.steps
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    rc = 0
+    for i in range(K):
+        a = i % nsets
+        rc |= lib.hsa_build_tree_fwd(*targs[a])
+        ev[i][0].record(stream)
+        rc |= lib.hsa_attn_fwd(*aargs[a])
+        ev[i][1].record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    assert rc == 0, lib.hsa_last_error()
+    ms_per_step = (t1 - t0) * 1e3 / K
+    attn_ms = sorted(a.elapsed_time(b) for a, b in ev)
+    attn_avg_ms = sum(attn_ms) / K
+    attn_med_ms = attn_ms[K // 2]
+
+    # --- the same K steps without events, and attention alone back to back ----------------
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        step(i)
+    torch.cuda.synchronize()
+    ms_per_step_noev = (time.perf_counter() - t0) * 1e3 / K
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(K):
+        lib.hsa_attn_fwd(*aargs[i % nsets])
+    e1.record(stream)
+    torch.cuda.synchronize()
+    attn_b2b_ms = e0.elapsed_time(e1) / K
+    e0.record(stream)
+    for i in range(K):
+        lib.hsa_build_tree_fwd(*targs[i % nsets])
+    e1.record(stream)
+    torch.cuda.synchronize()
+    tree_b2b_ms = e0.elapsed_time(e1) / K
+
+    head_queries = B * N * H
+    attn_bytes = e * B * H * D * (N + 2 * M + N)             # Q + K_full + V_full + Out
+    tree_bytes = e * B * H * D * (3 * (N - 1) + 2 * N + 2 * (N - 1))  # Qp,Kp,Vp + leaves + two copies out
+    achieved = attn_bytes / (attn_avg_ms * 1e-3) / 1e9
+    result = {
+        "metric": "attn fwd queries/sec + % HBM roofline, B8 H8 N2048 d64 bf16 SWA16",
+        "value": head_queries / (ms_per_step * 1e-3),
+        "unit": "head-queries/s",
+        "n_gpus": 1, "steps": K, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "%s: %s; step = tree build + span attention forward" % (args.workload, desc),
+                   "B": B, "H": H, "N": N, "D": D, "window_radius": R, "causal": causal,
+                   "buffer_sets_rotated": nsets, "bytes_per_set": set_bytes},
+        "roofline": {"bound": "hbm", "kernel": "attn_tile_kernel (span attention forward)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_ms": attn_avg_ms,
+                     "median_launch_ms": attn_med_ms},
+        "detail": {"attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
+                   "attn_back_to_back_ms": attn_b2b_ms, "tree_back_to_back_ms": tree_b2b_ms,
+                   "tree_algorithmic_bytes": tree_bytes,
+                   "tree_GBps_back_to_back": tree_bytes / (tree_b2b_ms * 1e-3) / 1e9,
+                   "attn_GBps_back_to_back": attn_bytes / (attn_b2b_ms * 1e-3) / 1e9,
+                   "ms_per_step_without_events": ms_per_step_noev},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(B, H, N, D, R, causal, scale, args.cpu_seconds)
+    if args.workload != "cfg3" or not causal:
+        result["metric"] = "attn fwd queries/sec + % HBM roofline, " + desc
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

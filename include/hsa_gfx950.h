@@ -103,12 +103,14 @@ int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const 
  *   qp, kp, vp  [B, N-1, H, D] level-concatenated (level 1 first, root last)
  *   k_leaf, v_leaf [B, N, H, D]
  *   out         [B, N-1, H, D] level-concatenated
+ *   out2        optional second copy of the result (NULL to skip), e.g. the node rows of
+ *               V_full when `out` is the node rows of K_full
  *   *_bs        batch strides in elements (0 = dense)
  */
 int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const void *k_leaf,
-                       const void *v_leaf, void *out, int B, int N, int H, int D, int64_t qp_bs,
-                       int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs,
-                       int64_t out_bs, int dtype, void *stream);
+                       const void *v_leaf, void *out, void *out2, int B, int N, int H, int D,
+                       int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs,
+                       int64_t vleaf_bs, int64_t out_bs, int64_t out2_bs, int dtype, void *stream);
 
 /*
  * Topology tables.  Replaces build_tree_topology

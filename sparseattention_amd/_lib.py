@@ -36,7 +36,7 @@ def _declare(lib):
     lib.hsa_attn_fwd_uses_tile.restype = I
     lib.hsa_build_parents_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 6 + [I, P]
     lib.hsa_build_parents_fwd.restype = I
-    lib.hsa_build_tree_fwd.argtypes = [P] * 6 + [I] * 4 + [I64] * 6 + [I, P]
+    lib.hsa_build_tree_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 7 + [I, P]
     lib.hsa_build_tree_fwd.restype = I
     lib.hsa_topology_host.argtypes = [I, I, P, P, P]
     lib.hsa_topology_host.restype = I

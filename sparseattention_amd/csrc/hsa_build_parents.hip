@@ -52,9 +52,9 @@ __global__ void __launch_bounds__(256)
 build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename T::storage *__restrict__ Kp,
                      const typename T::storage *__restrict__ Vp, const typename T::storage *__restrict__ Kc,
                      const typename T::storage *__restrict__ Vc, typename T::storage *__restrict__ Out,
-                     typename T::storage *__restrict__ Wt, int B, int P, int H, int D, int G,
-                     int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs,
-                     int64_t out_bs, float scale) {
+                     typename T::storage *__restrict__ Out2, typename T::storage *__restrict__ Wt, int B,
+                     int P, int H, int D, int G, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
+                     int64_t vc_bs, int64_t out_bs, int64_t out2_bs, float scale) {
     const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long unit = tid / G;
     const int gl = (int)(tid % G);
@@ -106,6 +106,7 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
     softmax3(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
     if (!active) return;
     typename T::storage *o = Out + (size_t)b * out_bs + prow;
+    typename T::storage *o2 = Out2 ? Out2 + (size_t)b * out2_bs + prow : nullptr;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int d = (c * G + gl) * VEC;
@@ -114,6 +115,7 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = w0 * fvp[c][e] + w1 * fv0[c][e] + w2 * fv1[c][e];
             store_vec<T, VEC>(o + d, r);
+            if (o2) store_vec<T, VEC>(o2 + d, r);
         }
     }
     if (Wt && gl == 0) {
@@ -126,9 +128,9 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
 
 template <typename T, int VEC>
 static int build_parents_launch(const void *qp, const void *kp, const void *vp, const void *kc,
-                                const void *vc, void *out, void *weights, int B, int P, int H, int D,
+                                const void *vc, void *out, void *out2, void *weights, int B, int P, int H, int D,
                                 int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs,
-                                int64_t out_bs, hipStream_t st) {
+                                int64_t out_bs, int64_t out2_bs, hipStream_t st) {
     using S = typename T::storage;
     const int chunks = (D + VEC - 1) / VEC;  // D % VEC == 0 guaranteed by the caller when VEC > 1
     int G = 1;
@@ -142,7 +144,7 @@ static int build_parents_launch(const void *qp, const void *kp, const void *vp, 
 #define HSA_BPN_LAUNCH(CHN)                                                                        \
     build_parents_kernel<T, VEC, CHN><<<(unsigned)blocks, block, 0, st>>>(                         \
         (const S *)qp, (const S *)kp, (const S *)vp, (const S *)kc, (const S *)vc, (S *)out,       \
-        (S *)weights, B, P, H, D, G, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, scale)
+        (S *)out2, (S *)weights, B, P, H, D, G, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, scale)
     if (CH == 1) HSA_BPN_LAUNCH(1);
     else if (CH == 2) HSA_BPN_LAUNCH(2);
     else if (CH <= 4) HSA_BPN_LAUNCH(4);
@@ -154,35 +156,36 @@ static int build_parents_launch(const void *qp, const void *kp, const void *vp, 
 
 template <typename T>
 static int build_parents_typed(const void *qp, const void *kp, const void *vp, const void *kc,
-                               const void *vc, void *out, void *weights, int B, int P, int H, int D,
-                               int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs,
-                               int64_t out_bs, hipStream_t st) {
+                               const void *vc, void *out, void *out2, void *weights, int B, int P, int H,
+                               int D, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
+                               int64_t vc_bs, int64_t out_bs, int64_t out2_bs, hipStream_t st) {
     constexpr int VEC = 16 / (int)sizeof(typename T::storage);
     const uintptr_t align = (uintptr_t)qp | (uintptr_t)kp | (uintptr_t)vp | (uintptr_t)kc | (uintptr_t)vc |
-                            (uintptr_t)out;
-    const int64_t strides = qp_bs | kp_bs | vp_bs | kc_bs | vc_bs | out_bs;
+                            (uintptr_t)out | (uintptr_t)out2;
+    const int64_t strides = qp_bs | kp_bs | vp_bs | kc_bs | vc_bs | out_bs | out2_bs;
     if (D % VEC == 0 && (align & 15) == 0 && (strides % VEC) == 0)
-        return build_parents_launch<T, VEC>(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs,
-                                            vp_bs, kc_bs, vc_bs, out_bs, st);
-    return build_parents_launch<T, 1>(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs, vp_bs,
-                                      kc_bs, vc_bs, out_bs, st);
+        return build_parents_launch<T, VEC>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs,
+                                            vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
+    return build_parents_launch<T, 1>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs,
+                                      kc_bs, vc_bs, out_bs, out2_bs, st);
 }
 
 int build_parents_dispatch(const void *qp, const void *kp, const void *vp, const void *kc, const void *vc,
-                           void *out, void *weights, int B, int P, int H, int D, int64_t qp_bs,
+                           void *out, void *out2, void *weights, int B, int P, int H, int D, int64_t qp_bs,
                            int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs, int64_t out_bs,
-                           int dtype, hipStream_t st) {
+                           int64_t out2_bs, int dtype, hipStream_t st) {
     const int64_t prow = (int64_t)P * H * D, crow = 2 * prow;
     if (!qp_bs) qp_bs = prow;
     if (!kp_bs) kp_bs = prow;
     if (!vp_bs) vp_bs = prow;
     if (!out_bs) out_bs = prow;
+    if (!out2_bs) out2_bs = prow;
     if (!kc_bs) kc_bs = crow;
     if (!vc_bs) vc_bs = crow;
     switch (dtype) {
-        case HSA_F32: return build_parents_typed<F32>(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, st);
-        case HSA_F16: return build_parents_typed<F16>(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, st);
-        case HSA_BF16: return build_parents_typed<BF16>(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, st);
+        case HSA_F32: return build_parents_typed<F32>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
+        case HSA_F16: return build_parents_typed<F16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
+        case HSA_BF16: return build_parents_typed<BF16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
     }
     return fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
 }
@@ -197,14 +200,14 @@ int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const 
                           int64_t out_bs, int dtype, void *stream) {
     HSA_REQUIRE(qp && kp && vp && kc && vc && out, "null pointer");
     HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
-    return hsa::build_parents_dispatch(qp, kp, vp, kc, vc, out, weights, B, P, H, D, qp_bs, kp_bs, vp_bs,
-                                       kc_bs, vc_bs, out_bs, dtype, (hipStream_t)stream);
+    return hsa::build_parents_dispatch(qp, kp, vp, kc, vc, out, nullptr, weights, B, P, H, D, qp_bs, kp_bs,
+                                       vp_bs, kc_bs, vc_bs, out_bs, 0, dtype, (hipStream_t)stream);
 }
 
 int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const void *k_leaf,
-                       const void *v_leaf, void *out, int B, int N, int H, int D, int64_t qp_bs,
+                       const void *v_leaf, void *out, void *out2, int B, int N, int H, int D, int64_t qp_bs,
                        int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs, int64_t out_bs,
-                       int dtype, void *stream) {
+                       int64_t out2_bs, int dtype, void *stream) {
     HSA_REQUIRE(qp && kp && vp && k_leaf && v_leaf && out, "null pointer");
     HSA_REQUIRE(B >= 1 && H >= 1 && D >= 1, "bad shape B=%d H=%d D=%d", B, H, D);
     HSA_REQUIRE(N >= 2 && hsa::ilog2_exact(N) >= 0, "N must be a power of two >= 2 (got %d)", N);
@@ -213,6 +216,7 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
     if (!kp_bs) kp_bs = tree;
     if (!vp_bs) vp_bs = tree;
     if (!out_bs) out_bs = tree;
+    if (!out2_bs) out2_bs = tree;
     if (!kleaf_bs) kleaf_bs = leaf;
     if (!vleaf_bs) vleaf_bs = leaf;
     const size_t es = hsa::elem_size(dtype);
@@ -224,8 +228,9 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
     for (int P = N / 2; P >= 1; P /= 2) {
         int rc = hsa::build_parents_dispatch((const char *)qp + off * row, (const char *)kp + off * row,
                                              (const char *)vp + off * row, kc, vc, (char *)out + off * row,
-                                             nullptr, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs,
-                                             dtype, (hipStream_t)stream);
+                                             out2 ? (char *)out2 + off * row : nullptr, nullptr, B, P, H, D,
+                                             qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, dtype,
+                                             (hipStream_t)stream);
         if (rc != HSA_OK) return rc;
         kc = vc = (const char *)out + off * row;
         kc_bs = vc_bs = out_bs;

@@ -46,7 +46,7 @@ def verify_tables(idx_table: torch.Tensor, mask_table: Optional[torch.Tensor]) -
 
 
 def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16,
-                      return_weights: bool = False, algo: str = "auto"):
+                      return_weights: bool = False, algo: str = "auto", out: Optional[torch.Tensor] = None):
     """Span attention forward on [B,N,H,D] / [B,M,H,D] tensors.
 
     Returns Out, or (Out, Weights [B,N,H,2R+1+L] fp32) with `return_weights`.
@@ -71,7 +71,10 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
     if canon is None and algo != "gather" and M >= 2 * N - 1:
         if verify_tables(idx_table, mask_table):
             canon = mask_table is not None
-    out = torch.empty_like(Q)
+    if out is None:
+        out = torch.empty_like(Q)
+    else:
+        assert out.shape == Q.shape and out.dtype == Q.dtype and out.is_contiguous() and out.is_cuda
     weights = (torch.empty((B, N, H, 2 * R + 1 + L), device=Q.device, dtype=torch.float32)
                if return_weights else None)
     lib = _lib.lib()
@@ -121,15 +124,17 @@ def _batch_stride(t: torch.Tensor) -> int:
     return t.stride(0) if B > 1 else rows * H * D
 
 
-def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None,
+               out2: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Every tree level in one call: level 1 from the leaves, level l+1 from level l's
     outputs used as both child keys and child values.
 
     Q_p, K_p, V_p [B, N-1, H, D] are level-concatenated (level 1 first, root last) and so
     is the result.  Tensors may be batch-strided slices of larger buffers (for instance
-    `out = K_full[:, N:]`) as long as each batch's rows are dense.
+    `out = K_full[:, N:]`) as long as each batch's rows are dense.  `out2`, if given,
+    receives a second copy of the result (for instance `V_full[:, N:]`).
     """
-    _lib.require_gpu(Q_p, K_p, V_p, K_leaf, V_leaf, out)
+    _lib.require_gpu(Q_p, K_p, V_p, K_leaf, V_leaf, out, out2)
     B, N, H, D = K_leaf.shape
     assert N >= 2 and (N & (N - 1)) == 0, "leaf count must be a power of 2"
     assert Q_p.shape == (B, N - 1, H, D) and K_p.shape == Q_p.shape and V_p.shape == Q_p.shape
@@ -137,6 +142,8 @@ def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None
     if out is None:
         out = torch.empty((B, N - 1, H, D), dtype=Q_p.dtype, device=Q_p.device)
     assert out.shape == Q_p.shape and out.dtype == Q_p.dtype
+    if out2 is not None:
+        assert out2.shape == Q_p.shape and out2.dtype == Q_p.dtype
     ts = [Q_p, K_p, V_p, K_leaf, V_leaf]
     for i, t in enumerate(ts):
         if not (t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D):
@@ -145,9 +152,9 @@ def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None
     with torch.cuda.device(Q_p.device):
         rc = _lib.lib().hsa_build_tree_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_leaf), _lib.ptr(V_leaf), _lib.ptr(out),
-            B, N, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
-            _batch_stride(K_leaf), _batch_stride(V_leaf), _batch_stride(out), _lib.dtype_code(Q_p),
-            _lib.stream_of(Q_p))
+            _lib.ptr(out2), B, N, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
+            _batch_stride(K_leaf), _batch_stride(V_leaf), _batch_stride(out),
+            _batch_stride(out2) if out2 is not None else 0, _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
     _lib.check(rc, "hsa_build_tree_fwd")
     return out
 

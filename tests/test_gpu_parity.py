@@ -168,8 +168,11 @@ def test_build_tree_vs_oracle(N, dtype):
     # writing straight into the node rows of a K_full buffer
     kfull = torch.zeros(B, 2 * N - 1, H, D, dtype=dtype, device=DEV)
     kfull[:, :N] = kl.to(DEV)
-    sa.build_tree(*(t.to(DEV) for t in (qp, kp, vp)), kfull[:, :N], vl.to(DEV), out=kfull[:, N:])
-    assert torch.equal(kfull[:, N:], out)
+    vfull = torch.zeros_like(kfull)
+    sa.build_tree(*(t.to(DEV) for t in (qp, kp, vp)), kfull[:, :N], vl.to(DEV), out=kfull[:, N:],
+                  out2=vfull[:, N:])
+    assert torch.equal(kfull[:, N:], out) and torch.equal(vfull[:, N:], out)
+    assert torch.equal(kfull[:, :N], kl.to(DEV)) and not vfull[:, :N].any()
 
 
 # ---------------------------------------------------------------- initial span nodes
@@ -289,8 +292,8 @@ def test_cfg3_headline_full_size(causal, bf):
     vfull = torch.empty_like(kfull)
     kfull[:, :N] = kl.to(DEV)
     vfull[:, :N] = vl.to(DEV)
-    sa.build_tree(qp.to(DEV), kp.to(DEV), vp.to(DEV), kfull[:, :N], vfull[:, :N], out=kfull[:, N:])
-    vfull[:, N:] = kfull[:, N:]
+    sa.build_tree(qp.to(DEV), kp.to(DEV), vp.to(DEV), kfull[:, :N], vfull[:, :N], out=kfull[:, N:],
+                  out2=vfull[:, N:])
     tree = oracle.build_tree_ref(qp, kp, vp, kl, vl, compute_dtype=torch.float64)
     assert_close(kfull[:, N:], tree, torch.bfloat16, "tree")
     t = sa.build_tree_topology(N, causal, device=DEV)
