@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 64 MiB -> 64 MiB copy kernel 10 times (reference for HBM counters)")
     return ap.parse_args()
 
 
@@ -175,6 +177,14 @@ def main():
     e1.record(stream)
     torch.cuda.synchronize()
     tree_b2b_ms = e0.elapsed_time(e1) / K
+
+    if args.calibrate_copy:
+        n = 64 * 2**20 // 2
+        src = [torch.randn(n, device=dev).to(torch.bfloat16) for _ in range(5)]
+        dst = [torch.empty(n, device=dev, dtype=torch.bfloat16) for _ in range(5)]
+        for i in range(10):
+            dst[i % 5].copy_(src[i % 5])
+        torch.cuda.synchronize()
 
     head_queries = B * N * H
     attn_bytes = e * B * H * D * (N + 2 * M + N)             # Q + K_full + V_full + Out

@@ -8,7 +8,9 @@
 //       the level-0 neighbour n^1 lies inside the block's own leaf block;
 //     - the 14 tree nodes of levels 1..3 under the block's level-4 ancestor
 //       (8 + 4 + 2 consecutive rows) and one sibling node per level 4..L-1, which is the
-//       same for all 16 queries: 14 + (L-4) <= 32 "tree slots" = two more key blocks.
+//       same for all 16 queries.  Levels 1..5 form a "near" key block that changes with
+//       every query block; levels 6..L-1 form a "far" key block that is the same for a
+//       whole aligned strip of up to 64 queries and is loaded once per strip.
 //   So the block's scores are a handful of dense 16x16 tiles with a per-element
 //   multiplicity mask (0: not attended, 1, or 2 for the leaf n^1 that is both a window
 //   key and the level-0 neighbour).
@@ -25,8 +27,9 @@
 // output channels of one query: the result is stored with one 16-byte store per 32
 // channels, in the same addressing pattern as the Q loads.
 // Leaf K / transposed-V operands slide along the strip in registers, so inside a strip
-// every K/V row is fetched once; the next block's operands are requested before the
-// current block is computed.
+// every K/V row is fetched once; later blocks' operands are requested before the current
+// block is computed (the strip loop is fully unrolled, every load has its own registers).
+// Lanes whose tree slot does not exist (level >= L) issue no load.
 #pragma once
 
 #include "hsa_common.h"
@@ -41,6 +44,7 @@ typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 template <typename T> struct Mma;
 
@@ -83,17 +87,17 @@ template <> struct Mma<F16> {
 };
 
 constexpr int TILE_Q = 16;           // queries per block
-constexpr int TILE_TREE_BLOCKS = 2;  // 32 tree slots
-constexpr int TILE_MAX_LEVELS = 22;  // 14 + (L - 4) <= 32
+constexpr int TILE_MAX_SB = 4;        // a strip is at most 64 aligned queries
+constexpr int TILE_MAX_LEVELS = 22;  // near block: levels 1..5, far block: levels 6..21
 constexpr float NEG_INF = -__builtin_inff();
 
 struct TileParams {
     const uint16_t *q, *k, *v;
     uint16_t *out;
     int B, N, M, H, L, R;
-    int SB;       // query blocks per strip
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
+    int xcd_swizzle;
     float scale_log2e;
 };
 
@@ -101,7 +105,10 @@ struct TileParams {
 // 4 (one per SIMD, <= 512 VGPRs) for 128 channels
 template <int D> constexpr int tile_max_wpb() { return D > 64 ? 4 : 8; }
 
-template <typename T, int D, int NBW, bool CAUSAL>
+// SB = query blocks per strip.  The strip loop is fully unrolled so that every load lands
+// in its own (virtual) registers: no loop-carried copies, the compiler's waits then cover
+// exactly the block being computed while later blocks' loads stay in flight.
+template <typename T, int D, int NBW, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(tile_max_wpb<D>() * 64)
 attn_tile_kernel(TileParams p) {
     using M_ = Mma<T>;
@@ -120,8 +127,9 @@ attn_tile_kernel(TileParams p) {
     // and upper tree nodes share an L2.
     int wg = blockIdx.x;
     const int nwg = gridDim.x;
-    if ((nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);
-    const int unit = wg * wpb + (threadIdx.x >> 6);
+    if (p.xcd_swizzle && (nwg & 7) == 0) wg = (wg & 7) * (nwg >> 3) + (wg >> 3);
+    // the wavefront index is the same in every lane: keep everything derived from it scalar
+    const int unit = wg * wpb + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (unit >= p.n_units) return;
     const int h = unit % p.H;
     const int s = (unit / p.H) % p.NS;
@@ -129,8 +137,7 @@ attn_tile_kernel(TileParams p) {
 
     const int N = p.N, L = p.L, R = p.R;
     const int NB = N / TILE_Q;
-    const int blk0 = s * p.SB;
-    const int nblk = (NB - blk0) < p.SB ? (NB - blk0) : p.SB;
+    const int blk0 = s * SB;  // NB is a multiple of SB (both powers of two, SB <= NB)
     const size_t rs = (size_t)p.H * D;  // elements between consecutive rows
     const uint16_t *Qb = p.q + ((size_t)b * N * p.H + h) * D + 8 * g;
     const uint16_t *Kb = p.k + ((size_t)b * p.M * p.H + h) * D + 8 * g;
@@ -168,57 +175,73 @@ attn_tile_kernel(TileParams p) {
         }
     }
 
-    // tree slots: slot s in [0,32).  0..7 level 1, 8..11 level 2, 12..13 level 3,
-    // 14+u level 4+u.  (a) the slot whose row this lane loads, per tree block;
-    // (b) level and liveness of the slots whose scores this lane holds.
-    int ld_off[TILE_TREE_BLOCKS], ld_lvl[TILE_TREE_BLOCKS], ld_add[TILE_TREE_BLOCKS], ld_xor[TILE_TREE_BLOCKS];
-#pragma unroll
-    for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
-        const int sl = 16 * t + r16;
-        int lvl, add, x;
-        if (sl < 8) { lvl = 1; add = sl; x = 0; }
-        else if (sl < 12) { lvl = 2; add = sl - 8; x = 0; }
-        else if (sl < 14) { lvl = 3; add = sl - 12; x = 0; }
-        else { lvl = 4 + (sl - 14); add = 0; x = 1; }
-        if (lvl >= L) { lvl = 1; add = 0; x = 0; }  // unused slot: point at a valid row
-        ld_lvl[t] = lvl; ld_add[t] = add; ld_xor[t] = x;
-        ld_off[t] = level_offset(N, lvl);
+    // tree slots.  Block T ("near", reloaded for every query block): slots 0..7 level 1,
+    // 8..11 level 2, 12..13 level 3 (the nodes under the block's level-4 ancestor), slot 14
+    // level 4, slot 15 level 5 (siblings of the ancestors).  Block U ("far", loaded once per
+    // strip): slot u is the sibling of the level-(6+u) ancestor, the same node for every
+    // query of an aligned 64-query strip.  Slots of levels >= L do not exist: not loaded.
+    int t_lvl, t_add, t_xor;   // the near slot whose row this lane loads
+    {
+        const int sl = r16;
+        if (sl < 8) { t_lvl = 1; t_add = sl; t_xor = 0; }
+        else if (sl < 12) { t_lvl = 2; t_add = sl - 8; t_xor = 0; }
+        else if (sl < 14) { t_lvl = 3; t_add = sl - 12; t_xor = 0; }
+        else { t_lvl = 4 + (sl - 14); t_add = 0; t_xor = 1; }
     }
-    float biasT[TILE_TREE_BLOCKS][4];   // constant part
-    int upT[TILE_TREE_BLOCKS][4];       // level of an upper slot (>= 4), or -1
+    const bool t_valid = t_lvl < L;
+    const int t_off = level_offset(N, t_lvl);
+    const int u_lvl = 6 + r16;
+    const bool u_valid = u_lvl < L;
+
+    float biasT[4];  // near block, constant part
+    int upT[4];      // level (4 or 5) of a near slot whose liveness depends on the block, or -1
 #pragma unroll
-    for (int t = 0; t < TILE_TREE_BLOCKS; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int sl = 16 * t + 4 * g + i;
-            int lvl, pl;
-            if (sl < 8) { lvl = 1; pl = sl; }
-            else if (sl < 12) { lvl = 2; pl = sl - 8; }
-            else if (sl < 14) { lvl = 3; pl = sl - 12; }
-            else { lvl = 4 + (sl - 14); pl = -1; }
-            bool live;
-            upT[t][i] = -1;
-            if (pl >= 0) {
-                live = pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1));
-            } else {
-                live = lvl < L;
-                if (CAUSAL && live) upT[t][i] = lvl;
-            }
-            biasT[t][i] = live ? 0.0f : NEG_INF;
+    for (int i = 0; i < 4; ++i) {
+        const int sl = 4 * g + i;
+        int lvl, pl;
+        if (sl < 8) { lvl = 1; pl = sl; }
+        else if (sl < 12) { lvl = 2; pl = sl - 8; }
+        else if (sl < 14) { lvl = 3; pl = sl - 12; }
+        else { lvl = 4 + (sl - 14); pl = -1; }
+        bool live;
+        upT[i] = -1;
+        if (pl >= 0) {
+            live = pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1));
+        } else {
+            live = lvl < L;
+            if (CAUSAL && live) upT[i] = lvl;
         }
+        biasT[i] = live ? 0.0f : NEG_INF;
+    }
+    const int qs = blk0 * TILE_Q;  // first query of the strip
+    float biasU[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int lvl = 6 + 4 * g + i;
+        const bool live = lvl < L && (!CAUSAL || ((qs >> lvl) & 1));
+        biasU[i] = live ? 0.0f : NEG_INF;
+    }
 
     // ---- loaders ----------------------------------------------------------------------
     auto load_rows = [&](const uint16_t *base, int row, uint4 (&dst)[KS]) {
         const uint16_t *ptr = base + (size_t)row * rs;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const uint4 *>(ptr + 32 * ks);
+        for (int ks = 0; ks < KS; ++ks) {
+#if defined(HSA_TILE_PROBE) && HSA_TILE_PROBE == 1   // timing probe: no loads
+            dst[ks] = make_uint4(0x3c003c00u + (uint32_t)row, 0x3c003c00u, 0x3c003c00u + (uint32_t)lane, 0x3c003c00u);
+#else
+            dst[ks] = *reinterpret_cast<const uint4 *>(ptr + 32 * ks);
+#endif
+        }
+    };
+    auto load_rows_if = [&](bool valid, const uint16_t *base, int row, uint4 (&dst)[KS]) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dst[ks] = make_uint4(0u, 0u, 0u, 0u);
+        if (valid) load_rows(base, row, dst);
     };
     auto leaf_row = [&](int kb) {  // first row of leaf block kb, clamped into the sequence
         kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
         return kb * TILE_Q + r16;
-    };
-    auto tree_row = [&](int t, int q0) {
-        return ld_off[t] + ((((q0 >> ld_lvl[t]) + ld_add[t])) ^ ld_xor[t]);
     };
     auto transpose_v = [&](const uint4 (&raw)[KS], uint2 (&dst)[NJ]) {
 #pragma unroll
@@ -229,7 +252,37 @@ attn_tile_kernel(TileParams p) {
         }
     };
 
-    // ---- rolling leaf operands ----------------------------------------------------------
+    // ---- per-block operand stage ----------------------------------------------------------
+    struct Stage {
+        uint4 q[KS], k[KS], v[KS], kt[KS], vt[KS];
+    };
+    auto request = [&](Stage &sg, int blk) {
+        const int q0 = blk * TILE_Q;
+        load_rows(Qb, q0 + r16, sg.q);
+        const int row = leaf_row(blk + (CAUSAL ? 0 : NBW));
+        load_rows(Kb, row, sg.k);
+        load_rows(Vb, row, sg.v);
+        const int tr = t_off + (((q0 >> t_lvl) + t_add) ^ t_xor);
+        load_rows_if(t_valid, Kb, tr, sg.kt);
+        load_rows_if(t_valid, Vb, tr, sg.vt);
+    };
+
+    // requests run AHEAD blocks in front of the computation
+    constexpr int AHEAD = (D <= 64) ? 2 : 1;
+    Stage st[SB];
+#pragma unroll
+    for (int i = 0; i < AHEAD && i < SB; ++i) request(st[i], blk0 + i);
+
+    // ---- per-strip operands: far tree block, leaf blocks left of the first query block ----
+    uint4 Ku[KS];
+    uint2 Vu[NJ];
+    {
+        const int ur = level_offset(N, u_valid ? u_lvl : 1) + ((qs >> u_lvl) ^ 1);
+        uint4 raw[KS];
+        load_rows_if(u_valid, Kb, ur, Ku);
+        load_rows_if(u_valid, Vb, ur, raw);
+        transpose_v(raw, Vu);
+    }
     uint4 Kl[NKL][KS];
     uint2 Vl[NKL][NJ];
 #pragma unroll
@@ -241,84 +294,84 @@ attn_tile_kernel(TileParams p) {
         transpose_v(raw, Vl[c]);
     }
 
-    // operands requested one block ahead
-    uint4 nQ[KS], nK[KS], nV[KS], nKt[TILE_TREE_BLOCKS][KS], nVt[TILE_TREE_BLOCKS][KS];
-    auto request = [&](int blk) {
+    auto process = [&](Stage &sg, int blk, Stage &nsg, int next_blk) {
         const int q0 = blk * TILE_Q;
-        load_rows(Qb, q0 + r16, nQ);
-        const int row = leaf_row(blk + (CAUSAL ? 0 : NBW));
-        load_rows(Kb, row, nK);
-        load_rows(Vb, row, nV);
+#if defined(HSA_TILE_PROBE) && HSA_TILE_PROBE == 2   // timing probe: loads and stores only
+        {
+            uint4 acc = make_uint4(0, 0, 0, 0);
 #pragma unroll
-        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
-            const int tr = tree_row(t, q0);
-            load_rows(Kb, tr, nKt[t]);
-            load_rows(Vb, tr, nVt[t]);
+            for (int ks = 0; ks < KS; ++ks) {
+                acc.x ^= sg.q[ks].x ^ sg.k[ks].y ^ sg.v[ks].z ^ sg.kt[ks].w ^ sg.vt[ks].x ^ Ku[ks].x ^ Kl[0][ks].x;
+                acc.y ^= sg.q[ks].y ^ sg.k[ks].x ^ sg.v[ks].w ^ sg.kt[ks].z ^ sg.vt[ks].y;
+            }
+            if (next_blk >= 0) request(nsg, next_blk);
+            uint16_t *optr = Ob + (size_t)(q0 + r16) * rs;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<uint4 *>(optr + 32 * ks) = acc;
+            return;
         }
-    };
-    request(blk0);
-
-    for (int it = 0; it < nblk; ++it) {
-        const int blk = blk0 + it;
-        const int q0 = blk * TILE_Q;
-        uint4 Qf[KS], Kt[TILE_TREE_BLOCKS][KS], rawV[KS], rawVt[TILE_TREE_BLOCKS][KS];
+#endif
+        // scores, transposed: acc[i] = <key 4g+i of the block, query r16>
+        f32x4 accL[NKL], accT, accU;
+#pragma unroll
+        for (int c = 0; c < NKL; ++c) {
+            accL[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                accL[c] = M_::k32(c == NEWC ? sg.k[ks] : Kl[c][ks], sg.q[ks], accL[c]);
+        }
+        accT = f32x4{0.f, 0.f, 0.f, 0.f};
+        accU = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            Qf[ks] = nQ[ks];
-            Kl[NEWC][ks] = nK[ks];
-            rawV[ks] = nV[ks];
-#pragma unroll
-            for (int t = 0; t < TILE_TREE_BLOCKS; ++t) { Kt[t][ks] = nKt[t][ks]; rawVt[t][ks] = nVt[t][ks]; }
+            accT = M_::k32(sg.kt[ks], sg.q[ks], accT);
+            accU = M_::k32(Ku[ks], sg.q[ks], accU);
         }
-        if (it + 1 < nblk) request(blk + 1);
+        // new value blocks into "lane = channel, regs = keys" form
+        uint2 Vt[NJ];
+        transpose_v(sg.v, Vl[NEWC]);
+        transpose_v(sg.vt, Vt);
+        if (NKL > 1) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) Kl[NEWC][ks] = sg.k[ks];
+        }
+        // this block's operands are consumed: request a later block's
+        if (next_blk >= 0) request(nsg, next_blk);
 
-        // scores, transposed: S[c][i] = score(key 4g+i of block c, query r16)
-        float sc[NKL + TILE_TREE_BLOCKS][4];
+        float sc[NKL + 2][4];
         float mx = NEG_INF;
 #pragma unroll
         for (int c = 0; c < NKL; ++c) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) acc = M_::k32(Kl[c][ks], Qf[ks], acc);
             const int kb = blk - NBW + c;
             const bool inside = kb >= 0 && kb < NB;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float v = inside ? fmaf(acc[i], p.scale_log2e, biasL[c][i]) : NEG_INF;
+                float v = inside ? fmaf(accL[c][i], p.scale_log2e, biasL[c][i]) : NEG_INF;
                 sc[c][i] = v;
                 mx = fmaxf(mx, v);
             }
         }
 #pragma unroll
-        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) acc = M_::k32(Kt[t][ks], Qf[ks], acc);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float bias = biasT[t][i];
-                if (CAUSAL) {
-                    const int lv = upT[t][i];
-                    if (lv >= 0 && ((q0 >> lv) & 1) == 0) bias = NEG_INF;
-                }
-                float v = fmaf(acc[i], p.scale_log2e, bias);
-                sc[NKL + t][i] = v;
-                mx = fmaxf(mx, v);
+        for (int i = 0; i < 4; ++i) {
+            float bias = biasT[i];
+            if (CAUSAL) {
+                const int lv = upT[i];
+                if (lv >= 0 && ((q0 >> lv) & 1) == 0) bias = NEG_INF;
             }
+            float v = fmaf(accT[i], p.scale_log2e, bias);
+            sc[NKL][i] = v;
+            mx = fmaxf(mx, v);
+            float u = fmaf(accU[i], p.scale_log2e, biasU[i]);
+            sc[NKL + 1][i] = u;
+            mx = fmaxf(mx, u);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
 
-        // new value blocks into "lane = channel, regs = keys" form
-        uint2 Vt[TILE_TREE_BLOCKS][NJ];
-        transpose_v(rawV, Vl[NEWC]);
-#pragma unroll
-        for (int t = 0; t < TILE_TREE_BLOCKS; ++t) transpose_v(rawVt[t], Vt[t]);
-
         float den = 0.f;
-        uint2 P[NKL + TILE_TREE_BLOCKS];
+        uint2 P[NKL + 2];
 #pragma unroll
-        for (int c = 0; c < NKL + TILE_TREE_BLOCKS; ++c) {
+        for (int c = 0; c < NKL + 2; ++c) {
             float e[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -341,12 +394,15 @@ attn_tile_kernel(TileParams p) {
                 f32x4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < NKL; ++c) o = M_::k16(Vl[c][j], P[c], o);
-#pragma unroll
-                for (int t = 0; t < TILE_TREE_BLOCKS; ++t) o = M_::k16(Vt[t][j], P[NKL + t], o);
+                o = M_::k16(Vt[j], P[NKL], o);
+                o = M_::k16(Vu[j], P[NKL + 1], o);
                 w[2 * jj] = M_::pack(o[0] * inv, o[1] * inv);
                 w[2 * jj + 1] = M_::pack(o[2] * inv, o[3] * inv);
             }
-            *reinterpret_cast<uint4 *>(optr + 32 * ks) = make_uint4(w[0], w[1], w[2], w[3]);
+            // the output is not read again by this kernel: streaming store (measured ~6% faster
+            // than a regular store on the 96 MiB headline shape)
+            __builtin_nontemporal_store(u32x4_t{w[0], w[1], w[2], w[3]},
+                                        reinterpret_cast<u32x4_t *>(optr + 32 * ks));
         }
 
         // slide the leaf window by one block
@@ -357,10 +413,16 @@ attn_tile_kernel(TileParams p) {
 #pragma unroll
             for (int j = 0; j < NJ; ++j) Vl[c][j] = Vl[c + 1][j];
         }
+    };
+
+#pragma unroll
+    for (int it = 0; it < SB; ++it) {
+        if (it + AHEAD < SB) process(st[it], blk0 + it, st[it + AHEAD], blk0 + it + AHEAD);
+        else process(st[it], blk0 + it, st[it], -1);
     }
 }
 
 template <typename T, int D>
-int attn_tile_launch_td(const TileParams &p, int nbw, bool causal, int wpb, hipStream_t st);
+int attn_tile_launch_td(const TileParams &p, int nbw, bool causal, int sb, int wpb, hipStream_t st);
 
 }  // namespace hsa

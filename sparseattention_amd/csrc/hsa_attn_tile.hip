@@ -32,26 +32,25 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     // strip length: long enough to amortise the halo and to prefetch, short enough to give
     // every SIMD of the 256 CUs at least two wavefronts
     const long block_units = (long)B * H * NB;
-    int sb = (int)(block_units / 2048);
-    if (sb < 1) sb = 1;
-    if (sb > 8) sb = 8;
-    if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x >= 1) sb = x; }
-    if (sb > NB) sb = NB;
-    p.SB = sb;
-    p.NS = (NB + sb - 1) / sb;
+    int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
+    if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+    while (sb > NB) sb >>= 1;  // NB is a power of two
+    p.NS = NB / sb;
     const long units = (long)B * p.NS * H;
     if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.n_units = (int)units;
+    p.xcd_swizzle = 1;
+    if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) p.xcd_swizzle = atoi(e);
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
     int wpb = 8;
     if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (dtype == HSA_BF16) {
-        if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, wpb, st);
-        return attn_tile_launch_td<BF16, 128>(p, nbw, causal != 0, wpb, st);
+        if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, sb, wpb, st);
+        return attn_tile_launch_td<BF16, 128>(p, nbw, causal != 0, sb, wpb, st);
     }
-    if (D == 64) return attn_tile_launch_td<F16, 64>(p, nbw, causal != 0, wpb, st);
-    return attn_tile_launch_td<F16, 128>(p, nbw, causal != 0, wpb, st);
+    if (D == 64) return attn_tile_launch_td<F16, 64>(p, nbw, causal != 0, sb, wpb, st);
+    return attn_tile_launch_td<F16, 128>(p, nbw, causal != 0, sb, wpb, st);
 }
 
 }  // namespace hsa

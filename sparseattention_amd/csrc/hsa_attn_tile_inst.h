@@ -5,25 +5,35 @@
 
 namespace hsa {
 
-template <typename T, int D, int NBW, bool CAUSAL>
+template <typename T, int D, int NBW, bool CAUSAL, int SB>
 static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
     if (wpb > tile_max_wpb<D>()) wpb = tile_max_wpb<D>();
     const int nwg = (p.n_units + wpb - 1) / wpb;
-    attn_tile_kernel<T, D, NBW, CAUSAL><<<nwg, wpb * 64, 0, st>>>(p);
+    attn_tile_kernel<T, D, NBW, CAUSAL, SB><<<nwg, wpb * 64, 0, st>>>(p);
     return check_launch("attn_tile_kernel");
+}
+
+template <typename T, int D, int NBW, bool CAUSAL>
+static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) {
+    switch (sb) {
+        case 1: return tile_launch_one<T, D, NBW, CAUSAL, 1>(p, wpb, st);
+        case 2: return tile_launch_one<T, D, NBW, CAUSAL, 2>(p, wpb, st);
+        case 4: return tile_launch_one<T, D, NBW, CAUSAL, 4>(p, wpb, st);
+    }
+    return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
 }
 
 #define HSA_TILE_INSTANTIATE(T, D)                                                              \
     template <>                                                                                 \
-    int attn_tile_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int wpb,          \
+    int attn_tile_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int sb, int wpb,  \
                                   hipStream_t st) {                                             \
         switch (nbw * 2 + (causal ? 1 : 0)) {                                                   \
-            case 0: return tile_launch_one<T, D, 0, false>(p, wpb, st);                         \
-            case 1: return tile_launch_one<T, D, 0, true>(p, wpb, st);                          \
-            case 2: return tile_launch_one<T, D, 1, false>(p, wpb, st);                         \
-            case 3: return tile_launch_one<T, D, 1, true>(p, wpb, st);                          \
-            case 4: return tile_launch_one<T, D, 2, false>(p, wpb, st);                         \
-            case 5: return tile_launch_one<T, D, 2, true>(p, wpb, st);                          \
+            case 0: return tile_launch_sb<T, D, 0, false>(p, sb, wpb, st);                      \
+            case 1: return tile_launch_sb<T, D, 0, true>(p, sb, wpb, st);                       \
+            case 2: return tile_launch_sb<T, D, 1, false>(p, sb, wpb, st);                      \
+            case 3: return tile_launch_sb<T, D, 1, true>(p, sb, wpb, st);                       \
+            case 4: return tile_launch_sb<T, D, 2, false>(p, sb, wpb, st);                      \
+            case 5: return tile_launch_sb<T, D, 2, true>(p, sb, wpb, st);                       \
         }                                                                                       \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel");       \
     }
