@@ -36,14 +36,28 @@ __device__ __forceinline__ void store_vec(typename T::storage *p, const float (&
     }
 }
 
-// 3-way softmax with the reference kernel's epsilon in the denominator.
+// 3-way softmax with the reference kernel's epsilon in the denominator.  fp32 tensors get
+// the accurate exp and division; 16-bit tensors (output precision 2^-9 or 2^-11) use the
+// hardware exp2 and reciprocal.
+template <typename T>
 __device__ __forceinline__ void softmax3(float s0, float s1, float s2, float &w0, float &w1, float &w2) {
     float m = fmaxf(s0, fmaxf(s1, s2));
-    float e0 = expf(s0 - m), e1 = expf(s1 - m), e2 = expf(s2 - m);
-    float den = e0 + e1 + e2 + 1e-9f;
-    w0 = e0 / den;
-    w1 = e1 / den;
-    w2 = e2 / den;
+    if constexpr (sizeof(typename T::storage) == 4) {
+        float e0 = expf(s0 - m), e1 = expf(s1 - m), e2 = expf(s2 - m);
+        float den = e0 + e1 + e2 + 1e-9f;
+        w0 = e0 / den;
+        w1 = e1 / den;
+        w2 = e2 / den;
+    } else {
+        constexpr float kLog2e = 1.4426950408889634f;
+        float e0 = __builtin_amdgcn_exp2f((s0 - m) * kLog2e);
+        float e1 = __builtin_amdgcn_exp2f((s1 - m) * kLog2e);
+        float e2 = __builtin_amdgcn_exp2f((s2 - m) * kLog2e);
+        float inv = __builtin_amdgcn_rcpf(e0 + e1 + e2 + 1e-9f);
+        w0 = e0 * inv;
+        w1 = e1 * inv;
+        w2 = e2 * inv;
+    }
 }
 
 // CH = number of VEC-chunks each lane holds (D <= G * VEC * CH).
@@ -97,13 +111,11 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
             load_vec<T, VEC>(v1 + d, fv1[c]);
         }
     }
-    for (int o = G >> 1; o >= 1; o >>= 1) {
-        s0 += __shfl_xor(s0, o, 64);
-        s1 += __shfl_xor(s1, o, 64);
-        s2 += __shfl_xor(s2, o, 64);
-    }
+    s0 = group_sum(s0, G);
+    s1 = group_sum(s1, G);
+    s2 = group_sum(s2, G);
     float w0, w1, w2;
-    softmax3(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
+    softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
     if (!active) return;
     typename T::storage *o = Out + (size_t)b * out_bs + prow;
     typename T::storage *o2 = Out2 ? Out2 + (size_t)b * out2_bs + prow : nullptr;
@@ -152,6 +164,217 @@ static int build_parents_launch(const void *qp, const void *kp, const void *vp, 
     else return fail(HSA_ERR_UNSUPPORTED, "head_dim %d too large", D);
 #undef HSA_BPN_LAUNCH
     return check_launch("build_parents_kernel");
+}
+
+// ---- several levels per launch ----------------------------------------------------------
+// A group of G lanes owns one (batch, head) and a subtree of 2^TL consecutive children
+// (leaves, or the outputs of the previous pass).  The children's K/V pieces and every
+// intermediate level stay in registers; each level's output is rounded to the element
+// type before it feeds the next level, exactly as if the levels had been separate calls.
+// With G * VEC == D a wavefront reads whole token rows (all heads) per load instruction.
+// SHARED: the children's keys and values are the same rows (every pass after the first),
+// loaded once.  Passes of four levels run one wavefront per workgroup (up to 512 VGPRs).
+template <int TL> constexpr int subtree_block() { return TL >= 4 ? 64 : 256; }
+
+template <typename T, int VEC, int TL, bool SHARED>
+__global__ void __launch_bounds__(subtree_block<TL>())
+build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename T::storage *__restrict__ Kp,
+                     const typename T::storage *__restrict__ Vp, const typename T::storage *__restrict__ Kc,
+                     const typename T::storage *__restrict__ Vc, typename T::storage *__restrict__ Out,
+                     typename T::storage *__restrict__ Out2, int B, int N, int H, int D, int G, int lvl0,
+                     int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs,
+                     int64_t out_bs, int64_t out2_bs, float scale) {
+    using S = typename T::storage;
+    constexpr int NC = 1 << TL;
+    // 32-bit index arithmetic (the launcher guarantees the thread count fits); G and the
+    // number of subtrees per sequence are powers of two
+    const int tid = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    const int lg = 31 - __builtin_clz(G);
+    const int unit = tid >> lg;
+    const int gl = tid & (G - 1);
+    const int n_sub = (N >> lvl0) >> TL;  // subtrees per (batch, head)
+    const int lsub = 31 - __builtin_clz(n_sub);
+    const int units = (B * H) << lsub;
+    const bool active = unit < units;
+    const int u = active ? unit : units - 1;
+    const int h = u % H;
+    const int bs = u / H;  // batch * n_sub + sub
+    const int sub = bs & (n_sub - 1);
+    const int b = bs >> lsub;
+    const int d = gl * VEC;
+    const bool dok = d < D;
+    const size_t rs = (size_t)H * D;
+    const size_t hd = (size_t)h * D + (dok ? d : 0);
+
+    // Every row this subtree needs is requested up front (children first, then the parent
+    // q/k/v rows of all TL levels): one memory round trip instead of one per level.
+    using P = Pack<T, VEC>;
+    P rck[NC], rcv[SHARED ? 1 : NC], rq[NC - 1], rk[NC - 1], rv[NC - 1];
+    {
+        const S *kc = Kc + (size_t)b * kc_bs + (size_t)sub * NC * rs + hd;
+        const S *vc = Vc + (size_t)b * vc_bs + (size_t)sub * NC * rs + hd;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            rck[c] = *reinterpret_cast<const P *>(kc + (size_t)c * rs);
+            if (!SHARED) rcv[c] = *reinterpret_cast<const P *>(vc + (size_t)c * rs);
+        }
+    }
+#pragma unroll
+    for (int j = 1; j <= TL; ++j) {
+        const int np = NC >> j;
+        const int base = NC - 2 * np;  // slot of this level's first parent: 0, NC/2, 3NC/4, ...
+        const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + (size_t)sub * np;
+        const S *q = Qp + (size_t)b * qp_bs + lrow * rs + hd;
+        const S *kp = Kp + (size_t)b * kp_bs + lrow * rs + hd;
+        const S *vp = Vp + (size_t)b * vp_bs + lrow * rs + hd;
+#pragma unroll
+        for (int i = 0; i < NC / 2; ++i) {
+            if (i < np) {
+                rq[base + i] = *reinterpret_cast<const P *>(q + (size_t)i * rs);
+                rk[base + i] = *reinterpret_cast<const P *>(kp + (size_t)i * rs);
+                rv[base + i] = *reinterpret_cast<const P *>(vp + (size_t)i * rs);
+            }
+        }
+    }
+
+    // keep every request ahead of the first use
+    __builtin_amdgcn_sched_barrier(0);
+
+    float ck[NC][VEC], cv[NC][VEC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            ck[c][e] = to_float<T>(rck[c].e[e]);
+            cv[c][e] = SHARED ? ck[c][e] : to_float<T>(rcv[c].e[e]);
+        }
+    }
+#pragma unroll
+    for (int j = 1; j <= TL; ++j) {
+        const int np = NC >> j;
+        const int base = NC - 2 * np;
+        const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + (size_t)sub * np;
+        S *o = Out + (size_t)b * out_bs + lrow * rs + hd;
+        S *o2 = Out2 ? Out2 + (size_t)b * out2_bs + lrow * rs + hd : nullptr;
+#pragma unroll
+        for (int i = 0; i < NC / 2; ++i) {
+            if (i < np) {
+                float fq[VEC], fk[VEC], fv[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    fq[e] = to_float<T>(rq[base + i].e[e]);
+                    fk[e] = to_float<T>(rk[base + i].e[e]);
+                    fv[e] = to_float<T>(rv[base + i].e[e]);
+                }
+                float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    s0 = fmaf(fq[e], fk[e], s0);
+                    s1 = fmaf(fq[e], ck[2 * i][e], s1);
+                    s2 = fmaf(fq[e], ck[2 * i + 1][e], s2);
+                }
+                if (!dok) { s0 = 0.f; s1 = 0.f; s2 = 0.f; }
+                s0 = group_sum(s0, G);
+                s1 = group_sum(s1, G);
+                s2 = group_sum(s2, G);
+                float w0, w1, w2;
+                softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
+                float r[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float x = w0 * fv[e] + w1 * cv[2 * i][e] + w2 * cv[2 * i + 1][e];
+                    r[e] = to_float<T>(from_float<T>(x));  // the stored value feeds the next level
+                }
+                if (active && dok) {
+                    store_vec<T, VEC>(o + (size_t)i * rs, r);
+                    if (o2) store_vec<T, VEC>(o2 + (size_t)i * rs, r);
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) { ck[i][e] = r[e]; cv[i][e] = r[e]; }
+            }
+        }
+    }
+}
+
+template <typename T, int VEC>
+static int build_subtree_launch(const void *qp, const void *kp, const void *vp, const void *kc,
+                                const void *vc, void *out, void *out2, int B, int N, int H, int D, int lvl0,
+                                int tl, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
+                                int64_t vc_bs, int64_t out_bs, int64_t out2_bs, hipStream_t st) {
+    using S = typename T::storage;
+    const int chunks = (D + VEC - 1) / VEC;
+    int G = 1;
+    while (G < chunks) G <<= 1;  // caller guarantees chunks <= 64
+    const long units = (long)B * ((N >> lvl0) >> tl) * H;
+    const long threads = units * G;
+    const int block = tl >= 4 ? subtree_block<4>() : subtree_block<1>();
+    const long blocks = (threads + block - 1) / block;
+    if (threads + block > 0x7fffffffL) return HSA_ERR_UNSUPPORTED;  // 32-bit indexing in the kernel
+    const float scale = 1.0f / sqrtf((float)D);
+    const bool shared = (kc == vc && kc_bs == vc_bs);
+#define HSA_SUBTREE(TLN, SH)                                                                        \
+    build_subtree_kernel<T, VEC, TLN, SH><<<(unsigned)blocks, block, 0, st>>>(                      \
+        (const S *)qp, (const S *)kp, (const S *)vp, (const S *)kc, (const S *)vc, (S *)out, (S *)out2, B, \
+        N, H, D, G, lvl0, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, scale)
+    if (tl == 4 && shared) HSA_SUBTREE(4, true);
+    else if (tl == 1 && shared) HSA_SUBTREE(1, true);
+    else if (tl == 2 && shared) HSA_SUBTREE(2, true);
+    else if (tl == 3 && shared) HSA_SUBTREE(3, true);
+    else if (tl == 1) HSA_SUBTREE(1, false);
+    else if (tl == 2) HSA_SUBTREE(2, false);
+    else if (tl == 3) HSA_SUBTREE(3, false);
+    else return fail(HSA_ERR_INVALID, "internal: bad subtree pass");
+#undef HSA_SUBTREE
+    return check_launch("build_subtree_kernel");
+}
+
+// Whole tree, up to three levels per launch.  Returns HSA_ERR_UNSUPPORTED when the shape
+// does not fit the subtree kernel (the caller then goes level by level).
+template <typename T>
+static int build_tree_typed(const void *qp, const void *kp, const void *vp, const void *k_leaf,
+                            const void *v_leaf, void *out, void *out2, int B, int N, int H, int D,
+                            int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs,
+                            int64_t out_bs, int64_t out2_bs, hipStream_t st) {
+    constexpr int VEC16 = 16 / (int)sizeof(typename T::storage);
+    const uintptr_t align = (uintptr_t)qp | (uintptr_t)kp | (uintptr_t)vp | (uintptr_t)k_leaf |
+                            (uintptr_t)v_leaf | (uintptr_t)out | (uintptr_t)out2;
+    const int64_t strides = qp_bs | kp_bs | vp_bs | kleaf_bs | vleaf_bs | out_bs | out2_bs;
+    const bool vec_ok = D % VEC16 == 0 && (align & 15) == 0 && (strides % VEC16) == 0;
+    const int vec = vec_ok ? VEC16 : 1;
+    if ((D + vec - 1) / vec > 64) return HSA_ERR_UNSUPPORTED;
+    const int L = ilog2_exact(N);
+    const size_t row = (size_t)H * D * sizeof(typename T::storage);
+    int lvl0 = 0;
+    while (lvl0 < L) {
+        // three levels from the leaves (keys and values are different rows), then four at a time
+        const int cap = lvl0 == 0 ? 3 : 4;
+        const int tl = L - lvl0 >= cap ? cap : L - lvl0;
+        const void *kc = k_leaf, *vc = v_leaf;
+        int64_t kc_bs = kleaf_bs, vc_bs = vleaf_bs;
+        if (lvl0 > 0) {
+            kc = vc = (const char *)out + (size_t)(level_offset(N, lvl0) - N) * row;
+            kc_bs = vc_bs = out_bs;
+        }
+        int rc = vec_ok ? build_subtree_launch<T, VEC16>(qp, kp, vp, kc, vc, out, out2, B, N, H, D, lvl0, tl,
+                                                         qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st)
+                        : build_subtree_launch<T, 1>(qp, kp, vp, kc, vc, out, out2, B, N, H, D, lvl0, tl, qp_bs,
+                                                     kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
+        if (rc != HSA_OK) return rc;
+        lvl0 += tl;
+    }
+    return HSA_OK;
+}
+
+int build_tree_dispatch(const void *qp, const void *kp, const void *vp, const void *k_leaf, const void *v_leaf,
+                        void *out, void *out2, int B, int N, int H, int D, int64_t qp_bs, int64_t kp_bs,
+                        int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs, int64_t out_bs, int64_t out2_bs,
+                        int dtype, hipStream_t st) {
+    switch (dtype) {
+        case HSA_F32: return build_tree_typed<F32>(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs, vp_bs, kleaf_bs, vleaf_bs, out_bs, out2_bs, st);
+        case HSA_F16: return build_tree_typed<F16>(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs, vp_bs, kleaf_bs, vleaf_bs, out_bs, out2_bs, st);
+        case HSA_BF16: return build_tree_typed<BF16>(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs, vp_bs, kleaf_bs, vleaf_bs, out_bs, out2_bs, st);
+    }
+    return fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
 template <typename T>
@@ -219,9 +442,16 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
     if (!out2_bs) out2_bs = tree;
     if (!kleaf_bs) kleaf_bs = leaf;
     if (!vleaf_bs) vleaf_bs = leaf;
+    HSA_REQUIRE(dtype == HSA_F32 || dtype == HSA_F16 || dtype == HSA_BF16, "unknown dtype %d", dtype);
+    {
+        int rc = hsa::build_tree_dispatch(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs, vp_bs,
+                                          kleaf_bs, vleaf_bs, out_bs, out2_bs, dtype, (hipStream_t)stream);
+        if (rc != HSA_ERR_UNSUPPORTED) return rc;
+    }
     const size_t es = hsa::elem_size(dtype);
     const size_t row = (size_t)H * D * es;
-    // level by level; each level reads the previous level's rows of `out`
+    // shapes the subtree kernel does not take: level by level; each level reads the previous
+    // level's rows of `out`
     const char *kc = (const char *)k_leaf, *vc = (const char *)v_leaf;
     int64_t kc_bs = kleaf_bs, vc_bs = vleaf_bs;
     size_t off = 0;

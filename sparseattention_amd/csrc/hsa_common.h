@@ -41,12 +41,26 @@ template <> __device__ __forceinline__ float from_float<F32>(float x) { return x
 template <> __device__ __forceinline__ uint16_t from_float<F16>(float x) {
     return __half_as_ushort(__float2half_rn(x));
 }
-// round-to-nearest-even, NaN kept quiet
+// round-to-nearest-even (the hardware conversion of gfx950)
 template <> __device__ __forceinline__ uint16_t from_float<BF16>(float x) {
-    uint32_t u = __float_as_uint(x);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+    return __builtin_bit_cast(uint16_t, static_cast<__bf16>(x));
+}
+
+// ---- cross-lane sums inside an aligned group of G lanes (G a power of two) --------------
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+// quad swaps, then mirrors inside 8 and 16 lanes (after the quads hold their sums, a mirror
+// brings in the other half's sum); wider groups cross the 16-lane rows with a shuffle
+__device__ __forceinline__ float group_sum(float v, int G) {
+    if (G >= 2) v += dpp_move<0xB1>(v);    // quad_perm [1,0,3,2]
+    if (G >= 4) v += dpp_move<0x4E>(v);    // quad_perm [2,3,0,1]
+    if (G >= 8) v += dpp_move<0x141>(v);   // row_half_mirror
+    if (G >= 16) v += dpp_move<0x140>(v);  // row_mirror
+    if (G >= 32) v += __shfl_xor(v, 16, 64);
+    if (G >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
 }
 
 static inline int elem_size(int dtype) { return dtype == HSA_F32 ? 4 : 2; }

@@ -154,10 +154,11 @@ def test_build_parents_child_count_assert():
         sa.build_parent_nodes(z, z, z, z, z)
 
 
-@pytest.mark.parametrize("N", [2, 4, 64, 512])
+@pytest.mark.parametrize("N,H,D", [(2, 4, 64), (4, 4, 64), (8, 1, 8), (16, 3, 20), (64, 4, 64), (128, 12, 64),
+                                   (512, 4, 64), (1024, 2, 128), (32, 1, 520)])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_build_tree_vs_oracle(N, dtype):
-    B, H, D = 2, 4, 64
+def test_build_tree_vs_oracle(N, H, D, dtype):
+    B = 2
     g = torch.Generator().manual_seed(N)
     qp, kp, vp = (torch.randn(B, N - 1, H, D, generator=g).to(dtype) for _ in range(3))
     kl, vl = (torch.randn(B, N, H, D, generator=g).to(dtype) for _ in range(2))
