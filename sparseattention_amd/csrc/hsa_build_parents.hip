@@ -328,6 +328,114 @@ static int build_subtree_launch(const void *qp, const void *kp, const void *vp, 
     return check_launch("build_subtree_kernel");
 }
 
+// ---- the top of the tree in one launch ------------------------------------------------------
+// One workgroup per (batch, head) finishes every remaining level once at most TOP_MAX_CHILDREN
+// nodes are left per sequence.  A group of G lanes owns one parent per level; the q/k/v rows
+// of all levels are requested at the start (they do not depend on the children), each level's
+// outputs go to global memory and, rounded to the element type, to LDS for the next level.
+constexpr int TOP_MAX_LEVELS = 8;
+constexpr int TOP_THREADS = 1024;
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(TOP_THREADS)
+build_top_kernel(const typename T::storage *__restrict__ Qp, const typename T::storage *__restrict__ Kp,
+                 const typename T::storage *__restrict__ Vp, typename T::storage *__restrict__ Out,
+                 typename T::storage *__restrict__ Out2, int N, int H, int D, int G, int lvl0, int nlev,
+                 int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t out_bs, int64_t out2_bs, float scale) {
+    using S = typename T::storage;
+    using P = Pack<T, VEC>;
+    extern __shared__ __align__(16) unsigned char top_lds[];
+    const int lg = 31 - __builtin_clz(G);
+    const int grp = threadIdx.x >> lg;  // parent slot
+    const int gl = threadIdx.x & (G - 1);
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int nc = N >> lvl0;  // children of the first level
+    const size_t rs = (size_t)H * D;
+    const size_t hd = (size_t)h * D + (size_t)gl * VEC;
+    const size_t row_bytes = (size_t)D * sizeof(S);
+    // ping-pong level buffers in LDS: [nc/2 rows] and [nc/4 rows]
+    unsigned char *buf0 = top_lds, *buf1 = top_lds + (size_t)(nc / 2) * row_bytes;
+
+    // parent rows are requested TOP_AHEAD levels before they are used (they do not depend on
+    // the children), which bounds the registers to a few levels' worth
+    constexpr int TOP_AHEAD = 3;
+    P rq[TOP_MAX_LEVELS], rk[TOP_MAX_LEVELS], rv[TOP_MAX_LEVELS], c0, c1;
+    auto request = [&](int j) {  // j = 1-based level of this pass
+        if (j <= nlev && grp < (nc >> j)) {
+            const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + grp;
+            rq[j - 1] = *reinterpret_cast<const P *>(Qp + (size_t)b * qp_bs + lrow * rs + hd);
+            rk[j - 1] = *reinterpret_cast<const P *>(Kp + (size_t)b * kp_bs + lrow * rs + hd);
+            rv[j - 1] = *reinterpret_cast<const P *>(Vp + (size_t)b * vp_bs + lrow * rs + hd);
+        }
+    };
+    if (grp < (nc >> 1)) {
+        const S *ch = Out + (size_t)b * out_bs + ((size_t)(level_offset(N, lvl0) - N) + 2 * grp) * rs + hd;
+        c0 = *reinterpret_cast<const P *>(ch);
+        c1 = *reinterpret_cast<const P *>(ch + rs);
+    }
+#pragma unroll
+    for (int j = 1; j <= TOP_AHEAD; ++j) request(j);
+    __builtin_amdgcn_sched_barrier(0);
+
+#pragma unroll
+    for (int j = 1; j <= TOP_MAX_LEVELS; ++j) {
+        if (j <= nlev) {
+            const int np = nc >> j;
+            unsigned char *src = (j & 1) ? buf1 : buf0;  // level j-1 outputs (j >= 2)
+            unsigned char *dst = (j & 1) ? buf0 : buf1;
+            if (j + TOP_AHEAD <= TOP_MAX_LEVELS) request(j + TOP_AHEAD);
+            if (grp < np) {
+                if (j >= 2) {
+                    c0 = *reinterpret_cast<const P *>(src + (size_t)(2 * grp) * row_bytes + (size_t)gl * VEC * sizeof(S));
+                    c1 = *reinterpret_cast<const P *>(src + (size_t)(2 * grp + 1) * row_bytes + (size_t)gl * VEC * sizeof(S));
+                }
+                float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float q = to_float<T>(rq[j - 1].e[e]);
+                    s0 = fmaf(q, to_float<T>(rk[j - 1].e[e]), s0);
+                    s1 = fmaf(q, to_float<T>(c0.e[e]), s1);
+                    s2 = fmaf(q, to_float<T>(c1.e[e]), s2);
+                }
+                s0 = group_sum(s0, G);
+                s1 = group_sum(s1, G);
+                s2 = group_sum(s2, G);
+                float w0, w1, w2;
+                softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
+                P r;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e)
+                    r.e[e] = from_float<T>(w0 * to_float<T>(rv[j - 1].e[e]) + w1 * to_float<T>(c0.e[e]) +
+                                           w2 * to_float<T>(c1.e[e]));
+                const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + grp;
+                *reinterpret_cast<P *>(Out + (size_t)b * out_bs + lrow * rs + hd) = r;
+                if (Out2) *reinterpret_cast<P *>(Out2 + (size_t)b * out2_bs + lrow * rs + hd) = r;
+                if (j < nlev)
+                    *reinterpret_cast<P *>(dst + (size_t)grp * row_bytes + (size_t)gl * VEC * sizeof(S)) = r;
+            }
+            if (j < nlev) __syncthreads();
+        }
+    }
+}
+
+template <typename T, int VEC>
+static int build_top_launch(const void *qp, const void *kp, const void *vp, void *out, void *out2, int B,
+                            int N, int H, int D, int lvl0, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs,
+                            int64_t out_bs, int64_t out2_bs, hipStream_t st) {
+    using S = typename T::storage;
+    const int G = D / VEC;
+    const int nc = N >> lvl0;
+    const int nlev = ilog2_exact(N) - lvl0;
+    const size_t lds = (size_t)(nc / 2 + nc / 4 + 1) * D * sizeof(S);
+    const float scale = 1.0f / sqrtf((float)D);
+    int threads = (nc / 2) * G;
+    if (threads < 64) threads = 64;
+    build_top_kernel<T, VEC><<<B * H, threads, lds, st>>>((const S *)qp, (const S *)kp, (const S *)vp, (S *)out,
+                                                          (S *)out2, N, H, D, G, lvl0, nlev, qp_bs, kp_bs, vp_bs,
+                                                          out_bs, out2_bs, scale);
+    return check_launch("build_top_kernel");
+}
+
 // Whole tree, up to three levels per launch.  Returns HSA_ERR_UNSUPPORTED when the shape
 // does not fit the subtree kernel (the caller then goes level by level).
 template <typename T>
@@ -346,6 +454,12 @@ static int build_tree_typed(const void *qp, const void *kp, const void *vp, cons
     const size_t row = (size_t)H * D * sizeof(typename T::storage);
     int lvl0 = 0;
     while (lvl0 < L) {
+        // once few enough nodes are left, one launch finishes the tree
+        if (lvl0 > 0 && vec_ok && D % VEC16 == 0 && ((D / VEC16) & (D / VEC16 - 1)) == 0 && D / VEC16 <= 64 &&
+            L - lvl0 <= TOP_MAX_LEVELS && (long)((N >> lvl0) / 2) * (D / VEC16) <= TOP_THREADS &&
+            (long)B * H <= 0x7fffffffL)
+            return build_top_launch<T, VEC16>(qp, kp, vp, out, out2, B, N, H, D, lvl0, qp_bs, kp_bs, vp_bs, out_bs,
+                                              out2_bs, st);
         // three levels from the leaves (keys and values are different rows), then four at a time
         const int cap = lvl0 == 0 ? 3 : 4;
         const int tl = L - lvl0 >= cap ? cap : L - lvl0;
