@@ -186,6 +186,15 @@ def main():
             dst[i % 5].copy_(src[i % 5])
         torch.cuda.synchronize()
 
+    # HBM bytes per launch of the attention kernel as counted by rocprofv3 --pmc FETCH_SIZE /
+    # WRITE_SIZE (scaled by a plain copy of known size); recorded under profiles/
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "attn_tile_%s_traffic.json" % args.workload)
+    if os.path.exists(tpath):
+        rec = json.load(open(tpath))
+        if rec.get("causal") == causal:
+            traffic = rec["traffic_bytes_per_launch"]
+
     head_queries = B * N * H
     attn_bytes = e * B * H * D * (N + 2 * M + N)             # Q + K_full + V_full + Out
     tree_bytes = e * B * H * D * (3 * (N - 1) + 2 * N + 2 * (N - 1))  # Qp,Kp,Vp + leaves + two copies out
@@ -202,7 +211,7 @@ def main():
                    "buffer_sets_rotated": nsets, "bytes_per_set": set_bytes},
         "roofline": {"bound": "hbm", "kernel": "attn_tile_kernel (span attention forward)",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_ms": attn_avg_ms},
         "detail": {"attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
                    "tree_build_avg_launch_ms": tree_b2b_ms,
