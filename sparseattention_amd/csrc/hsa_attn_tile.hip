@@ -34,6 +34,7 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     const long block_units = (long)B * H * NB;
     int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
     if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+    if (!causal && (R + TILE_Q - 1) / TILE_Q >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
     while (sb > NB) sb >>= 1;  // NB is a power of two
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;

@@ -360,16 +360,21 @@ build_top_kernel(const typename T::storage *__restrict__ Qp, const typename T::s
     // the children), which bounds the registers to a few levels' worth
     constexpr int TOP_AHEAD = 3;
     P rq[TOP_MAX_LEVELS], rk[TOP_MAX_LEVELS], rv[TOP_MAX_LEVELS], c0, c1;
+    // Loads are unconditional (idle groups re-read the level's last row, levels past the root
+    // re-read the root's): a load under a lane-dependent branch would be waited for at the end
+    // of its branch, one memory round trip per level.
     auto request = [&](int j) {  // j = 1-based level of this pass
-        if (j <= nlev && grp < (nc >> j)) {
-            const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + grp;
-            rq[j - 1] = *reinterpret_cast<const P *>(Qp + (size_t)b * qp_bs + lrow * rs + hd);
-            rk[j - 1] = *reinterpret_cast<const P *>(Kp + (size_t)b * kp_bs + lrow * rs + hd);
-            rv[j - 1] = *reinterpret_cast<const P *>(Vp + (size_t)b * vp_bs + lrow * rs + hd);
-        }
+        const int je = j <= nlev ? j : nlev;
+        const int np = nc >> je;
+        const size_t lrow = (size_t)(level_offset(N, lvl0 + je) - N) + (grp < np ? grp : np - 1);
+        rq[j - 1] = *reinterpret_cast<const P *>(Qp + (size_t)b * qp_bs + lrow * rs + hd);
+        rk[j - 1] = *reinterpret_cast<const P *>(Kp + (size_t)b * kp_bs + lrow * rs + hd);
+        rv[j - 1] = *reinterpret_cast<const P *>(Vp + (size_t)b * vp_bs + lrow * rs + hd);
     };
-    if (grp < (nc >> 1)) {
-        const S *ch = Out + (size_t)b * out_bs + ((size_t)(level_offset(N, lvl0) - N) + 2 * grp) * rs + hd;
+    {
+        const int np = nc >> 1;
+        const S *ch = Out + (size_t)b * out_bs +
+                      ((size_t)(level_offset(N, lvl0) - N) + 2 * (grp < np ? grp : np - 1)) * rs + hd;
         c0 = *reinterpret_cast<const P *>(ch);
         c1 = *reinterpret_cast<const P *>(ch + rs);
     }
@@ -413,7 +418,13 @@ build_top_kernel(const typename T::storage *__restrict__ Qp, const typename T::s
                 if (j < nlev)
                     *reinterpret_cast<P *>(dst + (size_t)grp * row_bytes + (size_t)gl * VEC * sizeof(S)) = r;
             }
-            if (j < nlev) __syncthreads();
+            if (j < nlev) {
+                // LDS-only barrier: __syncthreads() would also drain the outstanding global loads
+                // (requested levels ahead on purpose) and stores
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+                __builtin_amdgcn_s_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            }
         }
     }
 }
