@@ -32,6 +32,9 @@ __device__ __forceinline__ void store_vec(typename T::storage *p, const float (&
         P v;
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v.e[i] = from_float<T>(f[i]);
+        static_assert(sizeof(P) == 16, "vector path moves 16 bytes per lane");
+        // regular store: the rows are read again by the next launch (a streaming store makes the
+        // tree build itself ~8% faster and the attention kernel after it as much slower)
         *reinterpret_cast<P *>(p) = v;
     }
 }
