@@ -32,7 +32,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=30)
-    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--noncausal", action="store_true")
     ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -76,6 +76,62 @@ def cpu_baseline(B, H, N, D, R, causal, scale, budget_s):
                       % (bs, B, cores, len(times))}
 
 
+def lm_forward_bench(args):
+    """cfg4: forward of the 6-layer decoder LM (d_model 512, 8 heads, FFN 2048 GELU, vocab 50257,
+    bf16, B=8, N=4096, window 16, random weights, token ids uniform over the vocabulary)."""
+    import torch
+    import sparseattention_amd as sa
+    from sparseattention_amd.ops import functional as fn
+    from sparseattention_amd.modules import attention as attn_mod
+
+    dev = torch.device("cuda:0")
+    B, N, V, d, H, ff, layers, R = 8, 4096, 50257, 512, 8, 2048, 6, 16
+    torch.manual_seed(0)
+    model = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation="gelu", max_len=N)
+    model = model.to(dev).to(torch.bfloat16).eval()
+    tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(0)).to(dev)
+    K = min(args.steps, 20)
+    with torch.no_grad():
+        for _ in range(3):
+            model(tok)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            model(tok)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / K
+        # time share of the two custom ops: the same forward with an event pair around each call
+        spans = {"build_parent_nodes": [], "hierarchical_attention": []}
+        orig_b, orig_h = attn_mod.build_parent_nodes, attn_mod.hierarchical_attention
+
+        def timed(name, f):
+            def g(*a, **k):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                r = f(*a, **k)
+                e1.record()
+                spans[name].append((e0, e1))
+                return r
+            return g
+
+        attn_mod.build_parent_nodes = timed("build_parent_nodes", orig_b)
+        attn_mod.hierarchical_attention = timed("hierarchical_attention", orig_h)
+        model(tok)
+        torch.cuda.synchronize()
+        attn_mod.build_parent_nodes, attn_mod.hierarchical_attention = orig_b, orig_h
+    share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
+    print(json.dumps({
+        "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
+        "value": B * N / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": 3,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "cfg4: decoder LM forward, random init, eval mode"},
+        "detail": {"ms_in_build_parent_nodes_event_pairs": share["build_parent_nodes"],
+                   "ms_in_hierarchical_attention_event_pairs": share["hierarchical_attention"],
+                   "calls_build_parent_nodes": len(spans["build_parent_nodes"]),
+                   "calls_hierarchical_attention": len(spans["hierarchical_attention"])}}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -86,6 +142,8 @@ def main():
     from sparseattention_amd import _lib
     import sparseattention_amd as sa
 
+    if args.workload == "cfg4":
+        return lm_forward_bench(args)
     B, H, N, D, R, scale, desc = WORKLOADS[args.workload]
     causal = not args.noncausal
     dev = torch.device("cuda:0")

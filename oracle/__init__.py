@@ -15,4 +15,5 @@ from .hsa_oracle import (  # noqa: F401
     topology_tables,
     update_x_from_y_ref,
 )
+from .lm_ref import lm_forward_ref  # noqa: F401
 from .bruteforce import BruteForce, build_bruteforce  # noqa: F401

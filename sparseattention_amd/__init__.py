@@ -14,7 +14,10 @@ from .ops import (  # noqa: F401,E402
     hierarchical_attention,
 )
 
+from .transformer import TransformerLM  # noqa: F401,E402
+
 __all__ = [
+    "TransformerLM",
     "HierarchicalAttention",
     "build_tree_topology",
     "generate_span_input_Y",

@@ -108,3 +108,17 @@ def test_module_state_dict_names():
     assert keys == {"Wq_y.weight", "Wk_y.weight", "Wv_y.weight", "out_proj_y.weight", "out_proj_y.bias",
                     "Wq_x.weight", "Wk_x.weight", "Wv_x.weight", "out_proj_x.weight", "out_proj_x.bias"}
     assert m._build_level_info(16) == ([8, 4, 2, 1], [0, 8, 12, 14])
+
+
+def test_transformer_lm_state_dict_layout():
+    m = sa.TransformerLM(50, 32, 4, 64, 1, dropout=0.0, max_len=64)
+    keys = set(m.state_dict().keys())
+    for k in ["embedding.weight", "pos_encoding.pe", "fc_out.weight", "fc_out.bias",
+              "layers.0.self_attn.Wq_y.weight", "layers.0.self_attn.out_proj_x.bias",
+              "layers.0.feed_forward.fc1.weight", "layers.0.norm_y.weight", "layers.0.alpha_proj.weight",
+              "layers.0.beta_proj.bias"]:
+        assert k in keys
+    assert m.fc_out.weight is m.embedding.weight
+    # a reference-style checkpoint with a DataParallel prefix loads
+    ck = {"model_state_dict": {"module." + k: v for k, v in m.state_dict().items()}}
+    m.load_reference_checkpoint(ck)

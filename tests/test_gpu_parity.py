@@ -304,3 +304,59 @@ def test_cfg3_headline_full_size(causal, bf):
     out_g = fn.attention_forward(q.to(DEV), kfull, vfull, t["forward_idx"],
                                  t["forward_mask"] if causal else None, R, algo="gather")
     assert (out.float() - out_g.float()).abs().max() < 2e-2
+
+
+# ---------------------------------------------------------------- the language model around the ops
+@pytest.mark.parametrize("activation", ["relu", "gelu"])
+def test_transformer_lm_vs_oracle(activation):
+    V, d, H, ff, layers, N, B, R = 211, 64, 4, 128, 2, 64, 2, 4
+    torch.manual_seed(1)
+    m = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation=activation, max_len=128).eval()
+    tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(2))
+    sd = {k: v.detach().clone() for k, v in m.state_dict().items()}
+    with torch.no_grad():
+        got = m.to(DEV)(tok.to(DEV))
+    want = oracle.lm_forward_ref(sd, tok, H, layers, R, activation)
+    assert got.shape == (B, N, V)
+    assert (got.double().cpu() - want).abs().max() < 2e-4
+
+
+# ---------------------------------------------------------------- long-sequence stress (size-independent checks)
+def test_cfg5_long_sequence_properties():
+    """B1 H16 N65536 D128 bf16 R32: too large for the gather oracle in seconds, so check what
+    the mathematics fixes plus a brute-force sample of rows."""
+    B, H, N, D, R = 1, 16, 65536, 128, 32
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, N, H, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, 2 * N - 1, H, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, 2 * N - 1, H, D, generator=g).to(torch.bfloat16)
+    t = sa.build_tree_topology(N, True, device=DEV)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    out = sa.hierarchical_attention(qd, kd, vd, t["forward_idx"], t["backward_gather"], t["forward_mask"], R)
+    # causal row 0 attends only itself
+    assert torch.equal(out[:, 0], vd[:, 0])
+    # constant values come back unchanged whatever the weights are
+    const = torch.full_like(vd, 0.5)
+    oc = sa.hierarchical_attention(qd, kd, const, t["forward_idx"], t["backward_gather"], t["forward_mask"], R)
+    assert (oc.float() - 0.5).abs().max() < 4e-3
+    # brute force on a sample of rows spread over the sequence (first, last, block borders)
+    rows = sorted(set([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 1023, 1024, 4095, 4096, 32767, 32768, 65534, 65535]
+                      + list(range(7, N, 4099))))
+    o = oracle.topology_tables(N, True)
+    sel = torch.tensor(rows)
+    outs = []
+    for n in rows:
+        L = o["forward_idx"].shape[1]
+        live = [int(o["forward_idx"][n, l]) for l in range(L) if not o["forward_mask"][n, l]]
+        keys = list(range(max(0, n - R), n + 1)) + live
+        qf = q[0, n].double()                      # [H, D]
+        kf = k[0, keys].double()                   # [S, H, D]
+        vf = v[0, keys].double()
+        s = torch.einsum("hd,shd->hs", qf, kf) / math.sqrt(D)
+        p = torch.softmax(s, dim=-1)
+        outs.append(torch.einsum("hs,shd->hd", p, vf))
+    want = torch.stack(outs).unsqueeze(0)
+    assert_close(out[:, sel], want, torch.bfloat16, "cfg5 sampled rows")
+    # the gather kernel agrees with the tile kernel at this size
+    og = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R, algo="gather")
+    assert (og.float() - out.float()).abs().max() < 2e-2
