@@ -131,6 +131,40 @@ int hsa_topology_device(int N, int causal, int32_t *idx, uint8_t *mask, int32_t 
  */
 int hsa_span_input_y(const void *x, void *y, int B, int N, int C, int dtype, void *stream);
 
+/*
+ * Backward of one parent-build level.
+ * Replaces BuildParentNodesFunc.backward + build_parent_nodes_backward_kernel
+ * (hierarchical_attention/ops/functional.py:66-111,
+ *  hierarchical_attention/ops/triton/build_parents.py:106-204).  The three weights are
+ * recomputed from the inputs, so the forward does not have to save them.
+ *   dout, qp, kp, vp, dqp, dkp, dvp  [B, P, H, D];  kc, vc, dkc, dvc  [B, 2P, H, D]; all dense.
+ */
+int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, const void *vp,
+                          const void *kc, const void *vc, void *dqp, void *dkp, void *dvp, void *dkc,
+                          void *dvc, int B, int P, int H, int D, int dtype, void *stream);
+
+/*
+ * Backward of the span attention for the canonical tables.
+ * Replaces HierarchicalAttentionFunc.backward and its five kernels
+ * (hierarchical_attention/ops/functional.py:171-264,
+ *  hierarchical_attention/ops/triton/sparse_attn.py:185-623): the per-query pass recomputes the
+ * weights and writes dQ plus the weights / dS workspaces, the per-key pass gathers dK and dV
+ * (fp32 accumulation, written once in the element type; rows that nobody attends get zeros).
+ *   q, dout, dq  [B, N, H, D];  k, v, dk, dv  [B, M, H, D], M >= 2N-1
+ *   ws_p, ws_ds  device float [B, N, H, 2R+1+L] each (workspace provided by the caller)
+ */
+int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                 void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
+                 int causal, int dtype, void *stream);
+
+/*
+ * Backward of the initial span nodes (the reference differentiates generate_span_input_Y,
+ * hierarchical_attention/ops/topology.py:153-169, through torch autograd):
+ *   dx[b, n, :] = sum_{l=1..log2 N} 2^-l * dy[b, level l node n >> l, :]
+ *   dy [B, N-1, C], dx [B, N, C]
+ */
+int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,427 @@
+// Backward passes of the two ops and of the initial span nodes.
+//
+//  parent build   one lane group per (batch, parent, head) recomputes the three weights from
+//                 q and the keys (nothing but the inputs has to be saved by the forward) and
+//                 writes every gradient row exactly once: children 2i, 2i+1 belong to parent i.
+//  span attention two launches, no atomics, deterministic:
+//                 (1) per (batch, query, head): recompute the slot weights P, form
+//                     dP_t = <dO, V_t>, dS_t = P_t (dP_t - sum_u P_u dP_u) / sqrt(D), store P and
+//                     dS (fp32, [B,N,H,2R+1+L], window slots first) and dQ = sum_t dS_t K_t;
+//                 (2) per (batch, key row, head): gather the queries that attend the row --
+//                     window neighbours and the level-0 sibling for a leaf, the 2^l leaves under
+//                     the sibling subtree for a level-l node -- and accumulate
+//                     dK = sum dS Q, dV = sum P dO in fp32, written once in the element type.
+//                 Canonical complete-binary-tree tables only.
+//  span nodes     dx[n] = sum_l 2^-l dY[level l, n >> l].
+#include "hsa_common.h"
+
+namespace hsa {
+
+// ---------------------------------------------------------------- parent build
+template <typename T, int VEC> struct BPack { typename T::storage e[VEC]; };
+
+template <typename T, int VEC>
+__device__ __forceinline__ void bload(const typename T::storage *p, float (&f)[VEC]) {
+    if constexpr (VEC == 1) {
+        f[0] = to_float<T>(p[0]);
+    } else {
+        BPack<T, VEC> v = *reinterpret_cast<const BPack<T, VEC> *>(p);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) f[i] = to_float<T>(v.e[i]);
+    }
+}
+template <typename T, int VEC>
+__device__ __forceinline__ void bstore(typename T::storage *p, const float (&f)[VEC]) {
+    if constexpr (VEC == 1) {
+        p[0] = from_float<T>(f[0]);
+    } else {
+        BPack<T, VEC> v;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v.e[i] = from_float<T>(f[i]);
+        *reinterpret_cast<BPack<T, VEC> *>(p) = v;
+    }
+}
+
+template <typename T, int VEC, int CH>
+__global__ void __launch_bounds__(256)
+build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typename T::storage *__restrict__ Qp,
+                         const typename T::storage *__restrict__ Kp, const typename T::storage *__restrict__ Vp,
+                         const typename T::storage *__restrict__ Kc, const typename T::storage *__restrict__ Vc,
+                         typename T::storage *__restrict__ dQ, typename T::storage *__restrict__ dKp,
+                         typename T::storage *__restrict__ dVp, typename T::storage *__restrict__ dKc,
+                         typename T::storage *__restrict__ dVc, int B, int P, int H, int D, int G, float scale) {
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long unit = tid / G;
+    const int gl = (int)(tid % G);
+    const long units = (long)B * P * H;
+    const bool active = unit < units;
+    const long u = active ? unit : units - 1;
+    const int h = (int)(u % H);
+    const int i = (int)((u / H) % P);
+    const int b = (int)(u / ((long)H * P));
+    const size_t prow = (((size_t)b * P + i) * H + h) * D;
+    const size_t c0row = (((size_t)b * 2 * P + 2 * i) * H + h) * D;
+    const size_t c1row = c0row + (size_t)H * D;
+
+    float q[CH][VEC], kp[CH][VEC], k0[CH][VEC], k1[CH][VEC], vp[CH][VEC], v0[CH][VEC], v1[CH][VEC], g[CH][VEC];
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, p0 = 0.f, p1 = 0.f, p2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int d = (c * G + gl) * VEC;
+        if (d < D) {
+            bload<T, VEC>(Qp + prow + d, q[c]);
+            bload<T, VEC>(Kp + prow + d, kp[c]);
+            bload<T, VEC>(Kc + c0row + d, k0[c]);
+            bload<T, VEC>(Kc + c1row + d, k1[c]);
+            bload<T, VEC>(Vp + prow + d, vp[c]);
+            bload<T, VEC>(Vc + c0row + d, v0[c]);
+            bload<T, VEC>(Vc + c1row + d, v1[c]);
+            bload<T, VEC>(dO + prow + d, g[c]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                s0 = fmaf(q[c][e], kp[c][e], s0);
+                s1 = fmaf(q[c][e], k0[c][e], s1);
+                s2 = fmaf(q[c][e], k1[c][e], s2);
+                p0 = fmaf(g[c][e], vp[c][e], p0);
+                p1 = fmaf(g[c][e], v0[c][e], p1);
+                p2 = fmaf(g[c][e], v1[c][e], p2);
+            }
+        }
+    }
+    s0 = group_sum(s0, G); s1 = group_sum(s1, G); s2 = group_sum(s2, G);
+    p0 = group_sum(p0, G); p1 = group_sum(p1, G); p2 = group_sum(p2, G);
+    s0 *= scale; s1 *= scale; s2 *= scale;
+    const float m = fmaxf(s0, fmaxf(s1, s2));
+    const float e0 = expf(s0 - m), e1 = expf(s1 - m), e2 = expf(s2 - m);
+    const float den = e0 + e1 + e2 + 1e-9f;
+    const float w0 = e0 / den, w1 = e1 / den, w2 = e2 / den;
+    const float dot = w0 * p0 + w1 * p1 + w2 * p2;
+    const float ds0 = w0 * (p0 - dot) * scale, ds1 = w1 * (p1 - dot) * scale, ds2 = w2 * (p2 - dot) * scale;
+    if (!active) return;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int d = (c * G + gl) * VEC;
+        if (d < D) {
+            float r[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = ds0 * kp[c][e] + ds1 * k0[c][e] + ds2 * k1[c][e];
+            bstore<T, VEC>(dQ + prow + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = ds0 * q[c][e];
+            bstore<T, VEC>(dKp + prow + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = ds1 * q[c][e];
+            bstore<T, VEC>(dKc + c0row + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = ds2 * q[c][e];
+            bstore<T, VEC>(dKc + c1row + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = w0 * g[c][e];
+            bstore<T, VEC>(dVp + prow + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = w1 * g[c][e];
+            bstore<T, VEC>(dVc + c0row + d, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) r[e] = w2 * g[c][e];
+            bstore<T, VEC>(dVc + c1row + d, r);
+        }
+    }
+}
+
+template <typename T>
+static int build_parents_bwd_typed(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
+                                   const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B,
+                                   int P, int H, int D, hipStream_t st) {
+    using S = typename T::storage;
+    constexpr int VEC16 = 16 / (int)sizeof(S);
+    const uintptr_t al = (uintptr_t)dout | (uintptr_t)qp | (uintptr_t)kp | (uintptr_t)vp | (uintptr_t)kc |
+                         (uintptr_t)vc | (uintptr_t)dqp | (uintptr_t)dkp | (uintptr_t)dvp | (uintptr_t)dkc |
+                         (uintptr_t)dvc;
+    const bool vec_ok = D % VEC16 == 0 && (al & 15) == 0;
+    const int vec = vec_ok ? VEC16 : 1;
+    const int chunks = (D + vec - 1) / vec;
+    int G = 1;
+    while (G < chunks && G < 64) G <<= 1;
+    const int CH = (chunks + G - 1) / G;
+    const long threads = (long)B * P * H * G;
+    const long blocks = (threads + 255) / 256;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    const float scale = 1.0f / sqrtf((float)D);
+#define HSA_BWD(VECN, CHN)                                                                                  \
+    build_parents_bwd_kernel<T, VECN, CHN><<<(unsigned)blocks, 256, 0, st>>>(                               \
+        (const S *)dout, (const S *)qp, (const S *)kp, (const S *)vp, (const S *)kc, (const S *)vc, (S *)dqp, \
+        (S *)dkp, (S *)dvp, (S *)dkc, (S *)dvc, B, P, H, D, G, scale)
+    if (vec_ok) {
+        if (CH == 1) HSA_BWD(VEC16, 1);
+        else if (CH == 2) HSA_BWD(VEC16, 2);
+        else return fail(HSA_ERR_UNSUPPORTED, "head_dim %d too large", D);
+    } else {
+        if (CH == 1) HSA_BWD(1, 1);
+        else if (CH == 2) HSA_BWD(1, 2);
+        else if (CH <= 4) HSA_BWD(1, 4);
+        else if (CH <= 8) HSA_BWD(1, 8);
+        else return fail(HSA_ERR_UNSUPPORTED, "head_dim %d too large", D);
+    }
+#undef HSA_BWD
+    return check_launch("build_parents_bwd_kernel");
+}
+
+// ---------------------------------------------------------------- span attention, pass 1
+constexpr int BWD_MAX_CHUNKS = 4;
+
+__device__ __forceinline__ float bwd_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float bwd_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_bwd_query_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ K,
+                      const typename T::storage *__restrict__ V, const typename T::storage *__restrict__ dO,
+                      typename T::storage *__restrict__ dQ, float *__restrict__ Pw, float *__restrict__ DS, int B,
+                      int N, int M, int H, int D, int L, int R, int causal, float scale) {
+    const int lane = threadIdx.x & 63;
+    const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= (long)B * N * H) return;
+    const int h = (int)(unit % H);
+    const int n = (int)((unit / H) % N);
+    const int b = (int)(unit / ((long)H * N));
+    const int Wn = 2 * R + 1, S = Wn + L;
+    const size_t rs = (size_t)H * D;
+    const typename T::storage *q = Q + (((size_t)b * N + n) * H + h) * D;
+    const typename T::storage *go = dO + (((size_t)b * N + n) * H + h) * D;
+    const typename T::storage *kb = K + (size_t)b * M * rs + (size_t)h * D;
+    const typename T::storage *vb = V + (size_t)b * M * rs + (size_t)h * D;
+
+    int row[BWD_MAX_CHUNKS];
+    float sc[BWD_MAX_CHUNKS], dp[BWD_MAX_CHUNKS];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < BWD_MAX_CHUNKS; ++c) {
+        const int t = c * 64 + lane;
+        int r = -1;
+        if (t < Wn) {
+            const int j = n + t - R;
+            if (j >= 0 && j < N && (!causal || j <= n)) r = j;
+        } else if (t < S) {
+            const int l = t - Wn;
+            if (!(causal && (((n >> l) & 1) == 0))) r = level_offset(N, l) + ((n >> l) ^ 1);
+        }
+        row[c] = r;
+        float s = -INFINITY, g = 0.f;
+        if (r >= 0) {
+            const typename T::storage *kr = kb + (size_t)r * rs;
+            const typename T::storage *vr = vb + (size_t)r * rs;
+            float a = 0.f;
+            for (int d = 0; d < D; ++d) {
+                a = fmaf(to_float<T>(q[d]), to_float<T>(kr[d]), a);
+                g = fmaf(to_float<T>(go[d]), to_float<T>(vr[d]), g);
+            }
+            s = a * scale;
+        }
+        sc[c] = s;
+        dp[c] = g;
+        mx = fmaxf(mx, s);
+    }
+    mx = bwd_wave_max(mx);
+    float den = 0.f;
+#pragma unroll
+    for (int c = 0; c < BWD_MAX_CHUNKS; ++c) {
+        sc[c] = row[c] >= 0 ? expf(sc[c] - mx) : 0.f;
+        den += sc[c];
+    }
+    den = fmaxf(bwd_wave_sum(den), 1.0e-5f);
+    float dot = 0.f;
+#pragma unroll
+    for (int c = 0; c < BWD_MAX_CHUNKS; ++c) {
+        sc[c] /= den;
+        dot += sc[c] * dp[c];
+    }
+    dot = bwd_wave_sum(dot);
+    float *pw = Pw + (((size_t)b * N + n) * H + h) * S;
+    float *ds = DS + (((size_t)b * N + n) * H + h) * S;
+#pragma unroll
+    for (int c = 0; c < BWD_MAX_CHUNKS; ++c) {
+        dp[c] = sc[c] * (dp[c] - dot) * scale;  // dS
+        const int t = c * 64 + lane;
+        if (t < S) { pw[t] = sc[c]; ds[t] = dp[c]; }
+    }
+    typename T::storage *o = dQ + (((size_t)b * N + n) * H + h) * D;
+    for (int d0 = 0; d0 < D; d0 += 64) {
+        const int d = d0 + lane;
+        float acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < BWD_MAX_CHUNKS; ++c) {
+            const int lim = S - c * 64 < 64 ? S - c * 64 : 64;
+            for (int t = 0; t < lim; ++t) {
+                const int r = __shfl(row[c], t, 64);
+                const float w = __shfl(dp[c], t, 64);
+                if (r >= 0 && d < D) acc = fmaf(w, to_float<T>(kb[(size_t)r * rs + d]), acc);
+            }
+        }
+        if (d < D) o[d] = from_float<T>(acc);
+    }
+}
+
+// ---------------------------------------------------------------- span attention, pass 2
+// One wavefront per (batch, key row, head); lanes own channels.
+template <typename T>
+__global__ void __launch_bounds__(256)
+attn_bwd_key_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ dO,
+                    const float *__restrict__ Pw, const float *__restrict__ DS,
+                    typename T::storage *__restrict__ dK, typename T::storage *__restrict__ dV, int B, int N, int M,
+                    int H, int D, int L, int R, int causal) {
+    const int lane = threadIdx.x & 63;
+    const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= (long)B * M * H) return;
+    const int h = (int)(unit % H);
+    const int row = (int)((unit / H) % M);
+    const int b = (int)(unit / ((long)H * M));
+    const int Wn = 2 * R + 1, S = Wn + L;
+    const size_t rs = (size_t)H * D;
+    const typename T::storage *qb = Q + (size_t)b * N * rs + (size_t)h * D;
+    const typename T::storage *gb = dO + (size_t)b * N * rs + (size_t)h * D;
+    const float *pw = Pw + (size_t)b * N * H * S + (size_t)h * S;
+    const float *ds = DS + (size_t)b * N * H * S + (size_t)h * S;
+    const size_t ws = (size_t)H * S;  // weights stride between queries
+    typename T::storage *ok = dK + (((size_t)b * M + row) * H + h) * D;
+    typename T::storage *ov = dV + (((size_t)b * M + row) * H + h) * D;
+
+    for (int d0 = 0; d0 < D; d0 += 64) {
+        const int d = d0 + lane;
+        const bool dok = d < D;
+        float ak = 0.f, av = 0.f;
+        auto add = [&](int n, int slot) {
+            const float w = pw[(size_t)n * ws + slot];
+            const float s = ds[(size_t)n * ws + slot];
+            if (dok) {
+                ak = fmaf(s, to_float<T>(qb[(size_t)n * rs + d]), ak);
+                av = fmaf(w, to_float<T>(gb[(size_t)n * rs + d]), av);
+            }
+        };
+        if (row < N) {
+            const int lo = causal ? row : (row - R < 0 ? 0 : row - R);
+            const int hi = row + R >= N ? N - 1 : row + R;
+            for (int n = lo; n <= hi; ++n) add(n, row - n + R);
+            if (L > 0) {
+                const int sib = row ^ 1;  // the query whose level-0 neighbour is this leaf
+                if (!causal || (sib & 1)) add(sib, Wn);
+            }
+        } else if (row < 2 * N - 2) {  // tree node below the root
+            int lvl = 1;
+            while (row >= level_offset(N, lvl + 1)) ++lvl;
+            const int pidx = row - level_offset(N, lvl);
+            if (!causal || (pidx & 1) == 0) {
+                const int first = (pidx ^ 1) << lvl;
+                for (int n = first; n < first + (1 << lvl); ++n) add(n, Wn + lvl);
+            }
+        }
+        if (dok) {
+            ok[d] = from_float<T>(ak);
+            ov[d] = from_float<T>(av);
+        }
+    }
+}
+
+template <typename T>
+static int attn_bwd_typed(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                          void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
+                          int causal, hipStream_t st) {
+    using S = typename T::storage;
+    const float scale = 1.0f / sqrtf((float)D);
+    long units = (long)B * N * H;
+    long blocks = (units + 3) / 4;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    attn_bwd_query_kernel<T><<<(unsigned)blocks, 256, 0, st>>>((const S *)q, (const S *)k, (const S *)v,
+                                                               (const S *)dout, (S *)dq, ws_p, ws_ds, B, N, M, H, D,
+                                                               L, R, causal, scale);
+    int rc = check_launch("attn_bwd_query_kernel");
+    if (rc != HSA_OK) return rc;
+    units = (long)B * M * H;
+    blocks = (units + 3) / 4;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    attn_bwd_key_kernel<T><<<(unsigned)blocks, 256, 0, st>>>((const S *)q, (const S *)dout, ws_p, ws_ds, (S *)dk,
+                                                             (S *)dv, B, N, M, H, D, L, R, causal);
+    return check_launch("attn_bwd_key_kernel");
+}
+
+// ---------------------------------------------------------------- initial span nodes
+template <typename T>
+__global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, typename T::storage *__restrict__ dX,
+                                  int B, int N, int C, int L) {
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t total = (size_t)B * N * C;
+    if (t >= total) return;
+    const int c = (int)(t % C);
+    const int n = (int)((t / C) % N);
+    const int b = (int)(t / ((size_t)C * N));
+    const typename T::storage *dy = dY + (size_t)b * (N - 1) * C + c;
+    float acc = 0.f, w = 1.f;
+    for (int l = 1; l <= L; ++l) {
+        w *= 0.5f;
+        acc = fmaf(w, to_float<T>(dy[(size_t)(level_offset(N, l) - N + (n >> l)) * C]), acc);
+    }
+    dX[t] = from_float<T>(acc);
+}
+
+}  // namespace hsa
+
+extern "C" {
+
+int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
+                          const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B, int P,
+                          int H, int D, int dtype, void *stream) {
+    HSA_REQUIRE(dout && qp && kp && vp && kc && vc && dqp && dkp && dvp && dkc && dvc, "null pointer");
+    HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case HSA_F32: return hsa::build_parents_bwd_typed<hsa::F32>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
+        case HSA_F16: return hsa::build_parents_bwd_typed<hsa::F16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
+        case HSA_BF16: return hsa::build_parents_bwd_typed<hsa::BF16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
+    }
+    return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk, void *dv,
+                 float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R, int causal,
+                 int dtype, void *stream) {
+    HSA_REQUIRE(q && k && v && dout && dq && dk && dv && ws_p && ws_ds, "null pointer");
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
+    HSA_REQUIRE(hsa::ilog2_exact(N) == L, "canonical table needs L == log2 N (N=%d L=%d)", N, L);
+    HSA_REQUIRE(M >= 2 * N - 1, "canonical table needs M >= 2N-1 (N=%d M=%d)", N, M);
+    HSA_REQUIRE(R >= 0, "bad R=%d", R);
+    if (2 * R + 1 + L > 64 * hsa::BWD_MAX_CHUNKS)
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "2R+1+L = %d slots exceeds %d", 2 * R + 1 + L, 64 * hsa::BWD_MAX_CHUNKS);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case HSA_F32: return hsa::attn_bwd_typed<hsa::F32>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
+        case HSA_F16: return hsa::attn_bwd_typed<hsa::F16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
+        case HSA_BF16: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
+    }
+    return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtype, void *stream) {
+    HSA_REQUIRE(dy && dx, "null pointer");
+    HSA_REQUIRE(B >= 1 && C >= 1, "bad shape B=%d C=%d", B, C);
+    HSA_REQUIRE(N >= 2 && hsa::ilog2_exact(N) >= 0, "N must be a power of two >= 2 (got %d)", N);
+    const int L = hsa::ilog2_exact(N);
+    const size_t total = (size_t)B * N * C;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case HSA_F32: hsa::span_y_bwd_kernel<hsa::F32><<<blocks, 256, 0, st>>>((const float *)dy, (float *)dx, B, N, C, L); break;
+        case HSA_F16: hsa::span_y_bwd_kernel<hsa::F16><<<blocks, 256, 0, st>>>((const uint16_t *)dy, (uint16_t *)dx, B, N, C, L); break;
+        case HSA_BF16: hsa::span_y_bwd_kernel<hsa::BF16><<<blocks, 256, 0, st>>>((const uint16_t *)dy, (uint16_t *)dx, B, N, C, L); break;
+        default: return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+    }
+    return hsa::check_launch("span_y_bwd_kernel");
+}
+
+}  // extern "C"

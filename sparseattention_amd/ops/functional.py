@@ -159,35 +159,76 @@ def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None
     return out
 
 
+def build_parents_backward(grad_out, Q_p, K_p, V_p, K_c, V_c):
+    """Gradients (dQ_p, dK_p, dV_p, dK_c, dV_c) of one parent-build level."""
+    _lib.require_gpu(grad_out, Q_p, K_p, V_p, K_c, V_c)
+    grad_out, Q_p, K_p, V_p, K_c, V_c = (t.contiguous() for t in (grad_out, Q_p, K_p, V_p, K_c, V_c))
+    B, P, H, D = Q_p.shape
+    dq, dkp, dvp = torch.empty_like(Q_p), torch.empty_like(K_p), torch.empty_like(V_p)
+    dkc, dvc = torch.empty_like(K_c), torch.empty_like(V_c)
+    with torch.cuda.device(Q_p.device):
+        rc = _lib.lib().hsa_build_parents_bwd(
+            _lib.ptr(grad_out), _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c),
+            _lib.ptr(dq), _lib.ptr(dkp), _lib.ptr(dvp), _lib.ptr(dkc), _lib.ptr(dvc), B, P, H, D,
+            _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
+    _lib.check(rc, "hsa_build_parents_bwd")
+    return dq, dkp, dvp, dkc, dvc
+
+
+def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool):
+    """Gradients (dQ, dK, dV) of the span attention for the canonical tables of N = Q.shape[1]."""
+    _lib.require_gpu(grad_out, Q, K, V)
+    grad_out, Q, K, V = (t.contiguous() for t in (grad_out, Q, K, V))
+    B, N, H, D = Q.shape
+    M = K.shape[1]
+    L = N.bit_length() - 1
+    R = int(window_size)
+    S = 2 * R + 1 + L
+    dq, dk, dv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    ws = torch.empty((2, B, N, H, S), device=Q.device, dtype=torch.float32)
+    with torch.cuda.device(Q.device):
+        rc = _lib.lib().hsa_attn_bwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(grad_out), _lib.ptr(dq),
+                                     _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws[0]), _lib.ptr(ws[1]), B, N, M, H, D,
+                                     L, R, int(bool(causal)), _lib.dtype_code(Q), _lib.stream_of(Q))
+    _lib.check(rc, "hsa_attn_bwd")
+    return dq, dk, dv
+
+
 class BuildParentNodesFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q_p, K_p, V_p, K_c, V_c):
-        need_grad = any(ctx.needs_input_grad)
-        if need_grad:
-            out, w = build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights=True)
-            ctx.save_for_backward(Q_p, K_p, V_p, K_c, V_c, w)
-            return out
+        # the backward recomputes the three weights, so only the inputs are kept
+        ctx.save_for_backward(Q_p, K_p, V_p, K_c, V_c)
         return build_parents_forward(Q_p, K_p, V_p, K_c, V_c)
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("build_parent_nodes: this build provides the forward pass only")
+        return build_parents_backward(grad_output, *ctx.saved_tensors)
 
 
 class HierarchicalAttentionFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q, K, V, idx_table, gather_table, mask_table=None, window_size=16):
-        need_grad = any(ctx.needs_input_grad[:3])
-        if need_grad:
-            out, w = attention_forward(Q, K, V, idx_table, mask_table, window_size, return_weights=True)
-            ctx.save_for_backward(Q, K, V, idx_table, gather_table, w, mask_table)
+        out = attention_forward(Q, K, V, idx_table, mask_table, window_size)
+        if any(ctx.needs_input_grad[:3]):
+            N = Q.shape[1]
+            canon = _is_canonical(idx_table, mask_table, N)
+            if canon is None and K.shape[1] >= 2 * N - 1 and verify_tables(idx_table, mask_table):
+                canon = mask_table is not None
+            ctx.canonical = canon
             ctx.window_size = int(window_size)
-            return out
-        return attention_forward(Q, K, V, idx_table, mask_table, window_size)
+            ctx.save_for_backward(Q, K, V)
+        return out
 
     @staticmethod
     def backward(ctx, grad_output):
-        raise NotImplementedError("hierarchical_attention: this build provides the forward pass only")
+        if ctx.canonical is None:
+            raise NotImplementedError(
+                "hierarchical_attention backward needs the tables of build_tree_topology "
+                "(the reference's backward kernels make the same assumption through gather_table)")
+        Q, K, V = ctx.saved_tensors
+        dq, dk, dv = attention_backward(grad_output, Q, K, V, ctx.window_size, ctx.canonical)
+        return dq, dk, dv, None, None, None, None
 
 
 def build_parent_nodes(Q_p, K_p, V_p, K_c, V_c):

@@ -69,6 +69,30 @@ def build_tree_topology(seq_len: int, is_causal: bool = True, device="cuda",
     return {"forward_idx": idx, "forward_mask": fmask, "backward_gather": gat}
 
 
+class _SpanInputY(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        B, N, C = x.shape
+        x = x.contiguous()
+        y = torch.empty((B, N - 1, C), dtype=x.dtype, device=x.device)
+        with torch.cuda.device(x.device):
+            rc = _lib.lib().hsa_span_input_y(_lib.ptr(x), _lib.ptr(y), B, N, C, _lib.dtype_code(x),
+                                             _lib.stream_of(x))
+        _lib.check(rc, "hsa_span_input_y")
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        B, M, C = dy.shape
+        dy = dy.contiguous()
+        dx = torch.empty((B, M + 1, C), dtype=dy.dtype, device=dy.device)
+        with torch.cuda.device(dy.device):
+            rc = _lib.lib().hsa_span_input_y_bwd(_lib.ptr(dy), _lib.ptr(dx), B, M + 1, C, _lib.dtype_code(dy),
+                                                 _lib.stream_of(dy))
+        _lib.check(rc, "hsa_span_input_y_bwd")
+        return dx
+
+
 def generate_span_input_Y(x: torch.Tensor) -> Optional[torch.Tensor]:
     """Initial span nodes: pairwise means level by level, [B, N, C] -> [B, N-1, C]."""
     B, N, C = x.shape
@@ -76,10 +100,5 @@ def generate_span_input_Y(x: torch.Tensor) -> Optional[torch.Tensor]:
         return None
     assert (N & (N - 1)) == 0, "sequence length must be a power of 2"
     _lib.require_gpu(x)
-    x = x.contiguous()
-    y = torch.empty((B, N - 1, C), dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
-        rc = _lib.lib().hsa_span_input_y(_lib.ptr(x), _lib.ptr(y), B, N, C, _lib.dtype_code(x),
-                                         _lib.stream_of(x))
-    _lib.check(rc, "hsa_span_input_y")
-    return y
+    _lib.dtype_code(x)
+    return _SpanInputY.apply(x)

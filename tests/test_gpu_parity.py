@@ -360,3 +360,97 @@ def test_cfg5_long_sequence_properties():
     # the gather kernel agrees with the tile kernel at this size
     og = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R, algo="gather")
     assert (og.float() - out.float()).abs().max() < 2e-2
+
+
+# ---------------------------------------------------------------- backward passes
+def _grad_close(got, want, dtype, what):
+    got = got.detach().double().cpu()
+    scale = max(1.0, float(want.abs().max()))
+    atol = 2e-5 if dtype == torch.float32 else 3e-2
+    err = float((got - want).abs().max())
+    assert err <= atol * scale, "%s: max abs err %.3e (scale %.2f, dtype %s)" % (what, err, scale, dtype)
+
+
+@pytest.mark.parametrize("case", [(2, 8, 2, 16, 2, None), (1, 64, 3, 32, 5, None), (2, 128, 4, 64, 16, None),
+                                  (1, 32, 2, 20, 0, None), (1, 16, 2, 16, 20, 40)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
+    B, N, H, D, R, M = case
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=7 * N + R, M=M)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(3)).to(dtype)
+    o = oracle.topology_tables(N, causal)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    ref = oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"] if causal else None, R)
+    ref.backward(go.double())
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    qd, kd, vd = (x.to(DEV).requires_grad_(True) for x in (q, k, v))
+    out = sa.hierarchical_attention(qd, kd, vd, t["forward_idx"], t["backward_gather"],
+                                    t["forward_mask"] if causal else None, R)
+    out.backward(go.to(DEV))
+    assert qd.grad.dtype == dtype and kd.grad.shape == k.shape
+    _grad_close(qd.grad, qr.grad, dtype, "dQ")
+    _grad_close(kd.grad, kr.grad, dtype, "dK")
+    _grad_close(vd.grad, vr.grad, dtype, "dV")
+
+
+def test_attention_backward_rejects_unknown_tables():
+    N = 16
+    q, k, v = make_qkv(1, N, 1, 16, torch.float32, seed=1, M=40)
+    idx = torch.randint(0, 40, (N, 4), dtype=torch.int32).to(DEV)
+    qd = q.to(DEV).requires_grad_(True)
+    out = sa.hierarchical_attention(qd, k.to(DEV), v.to(DEV), idx, None, None, 2)
+    with pytest.raises(NotImplementedError):
+        out.sum().backward()
+
+
+@pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_build_parents_backward_vs_oracle_autograd(shape, dtype):
+    B, P, H, D = shape
+    g = torch.Generator().manual_seed(P + D)
+    qp, kp, vp = (torch.randn(B, P, H, D, generator=g).to(dtype) for _ in range(3))
+    kc, vc = (torch.randn(B, 2 * P, H, D, generator=g).to(dtype) for _ in range(2))
+    go = torch.randn(B, P, H, D, generator=g).to(dtype)
+    refs = [t.double().requires_grad_(True) for t in (qp, kp, vp, kc, vc)]
+    oracle.build_parent_nodes_ref(*refs).backward(go.double())
+    devs = [t.to(DEV).requires_grad_(True) for t in (qp, kp, vp, kc, vc)]
+    sa.build_parent_nodes(*devs).backward(go.to(DEV))
+    for name, d, r in zip(["dQp", "dKp", "dVp", "dKc", "dVc"], devs, refs):
+        _grad_close(d.grad, r.grad, dtype, name)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_span_input_y_backward(dtype):
+    B, N, C = 2, 64, 24
+    x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(0)).to(dtype)
+    gy = torch.randn(B, N - 1, C, generator=torch.Generator().manual_seed(1)).to(dtype)
+    xr = x.double().requires_grad_(True)
+    oracle.span_input_y_ref(xr).backward(gy.double())
+    xd = x.to(DEV).requires_grad_(True)
+    sa.generate_span_input_Y(xd).backward(gy.to(DEV))
+    _grad_close(xd.grad, xr.grad, dtype, "dx")
+
+
+def test_module_trains_end_to_end_like_the_oracle():
+    """One backward through cross_update_Y + forward of the module: parameter and input
+    gradients against autograd through the CPU oracle with the same weights."""
+    B, N, dim, H, R = 2, 32, 64, 4, 3
+    torch.manual_seed(0)
+    m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=R)
+    x = torch.randn(B, N, dim).clamp(-1, 1)
+    y = torch.randn(B, N - 1, dim).clamp(-1, 1)
+    w = {k: v.detach().double().requires_grad_(True) for k, v in m.state_dict().items()}
+    xr, yr = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    y2 = oracle.cross_update_y_ref(xr, yr, w, H)
+    ref = oracle.update_x_from_y_ref(xr, y2, w, H, R, causal=True)
+    ref.square().sum().backward()
+    md = m.to(DEV)
+    xd, yd = x.to(DEV).requires_grad_(True), y.to(DEV).requires_grad_(True)
+    out = md(xd, xd, xd, y=md.cross_update_Y(xd, yd), mask=torch.ones(1, device=DEV))
+    out.square().sum().backward()
+    assert (out.detach().double().cpu() - ref.detach()).abs().max() < 1e-4
+    _grad_close(xd.grad, xr.grad, torch.float32, "dx")
+    _grad_close(yd.grad, yr.grad, torch.float32, "dy")
+    for name, p in md.named_parameters():
+        _grad_close(p.grad, w[name].grad, torch.float32, name)

@@ -236,3 +236,19 @@ def test_module_compositions_reduce_to_ops():
         xy = torch.cat([x, y], 1).view(B, 2 * N - 1, H, Dh)
         want = oracle.attention_ref(xh, xy, xy, t["forward_idx"], t["forward_mask"] if causal else None, R)
         assert torch.allclose(got, want.reshape(B, N, D), atol=1e-6)
+
+
+def test_oracle_gradients_are_true_derivatives():
+    """The backward parity tests differentiate the oracle with autograd; check that against
+    finite differences on tiny fp64 problems."""
+    g = torch.Generator().manual_seed(0)
+    B, N, H, D, R = 1, 8, 1, 4, 2
+    q = torch.randn(B, N, H, D, generator=g, dtype=torch.float64, requires_grad=True)
+    k = torch.randn(B, 2 * N - 1, H, D, generator=g, dtype=torch.float64, requires_grad=True)
+    v = torch.randn(B, 2 * N - 1, H, D, generator=g, dtype=torch.float64, requires_grad=True)
+    t = oracle.topology_tables(N, True)
+    f = lambda a, b, c: oracle.attention_ref(a, b, c, t["forward_idx"], t["forward_mask"], R)
+    assert torch.autograd.gradcheck(f, (q, k, v), eps=1e-6, atol=1e-6)
+    qp, kp, vp = (torch.randn(1, 2, 1, 4, generator=g, dtype=torch.float64, requires_grad=True) for _ in range(3))
+    kc, vc = (torch.randn(1, 4, 1, 4, generator=g, dtype=torch.float64, requires_grad=True) for _ in range(2))
+    assert torch.autograd.gradcheck(oracle.build_parent_nodes_ref, (qp, kp, vp, kc, vc), eps=1e-6, atol=1e-6)
