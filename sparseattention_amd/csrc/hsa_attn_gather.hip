@@ -120,6 +120,165 @@ attn_gather_kernel(const typename T::storage *__restrict__ Q, const typename T::
     }
 }
 
+// ---- vector variant ---------------------------------------------------------------------------
+// D/VEC lanes (VEC = 16 bytes of elements) share one attention slot and read its key / value row
+// as one contiguous piece, so a wavefront covers SPW = 64*VEC/D slots per pass and every load is
+// a whole head-row.  Each lane keeps its VEC channels of q and of the output accumulator; scores
+// are reduced inside the lane group, the output across the SPW groups at the end.
+constexpr int GATHER_MAX_PASSES = 40;
+
+template <typename T, int VEC, int LPS /* lanes per slot = D / VEC */>
+__global__ void __launch_bounds__(256)
+attn_gather_vec_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ K,
+                       const typename T::storage *__restrict__ V, const int32_t *__restrict__ idx,
+                       const uint8_t *__restrict__ mask, typename T::storage *__restrict__ Out,
+                       float *__restrict__ W, int B, int N, int M, int H, int L, int R, int causal, float scale) {
+    constexpr int D = VEC * LPS;
+    constexpr int SPW = 64 / LPS;  // slots per pass
+    struct alignas(16) Pk { typename T::storage e[VEC]; };
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPS;    // slot inside a pass
+    const int gl = lane % LPS;     // channel piece
+    const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= (long)B * N * H) return;
+    const int h = (int)(unit % H);
+    const int n = (int)((unit / H) % N);
+    const int b = (int)(unit / ((long)H * N));
+    const int Wn = 2 * R + 1, S = Wn + L;
+    const int passes = (S + SPW - 1) / SPW;
+    const size_t rs = (size_t)H * D;
+    const typename T::storage *kb = K + (size_t)b * M * rs + (size_t)h * D + gl * VEC;
+    const typename T::storage *vb = V + (size_t)b * M * rs + (size_t)h * D + gl * VEC;
+
+    float q[VEC];
+    {
+        Pk t = *reinterpret_cast<const Pk *>(Q + (((size_t)b * N + n) * H + h) * D + gl * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) q[e] = to_float<T>(t.e[e]) * scale;
+    }
+    auto slot_row = [&](int t) {
+        int r = -1;
+        if (t < Wn) {
+            const int j = n + t - R;
+            if (j >= 0 && j < N && (!causal || j <= n)) r = j;
+        } else if (t < S) {
+            const int l = t - Wn;
+            if (idx) {
+                const int m = idx[(size_t)n * L + l];
+                if (m != -1 && !(mask && mask[(size_t)n * L + l] != 0)) r = m;
+            } else if (!(causal && (((n >> l) & 1) == 0))) {
+                r = level_offset(N, l) + ((n >> l) ^ 1);
+            }
+        }
+        return r;
+    };
+    // pass 1: scores of this lane group's slots (kept in registers, GATHER_MAX_PASSES bound)
+    float sc[GATHER_MAX_PASSES];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
+        sc[p] = -INFINITY;
+        if (p < passes) {
+            const int r = slot_row(p * SPW + sub);
+            if (r >= 0) {
+                Pk t = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
+                float a = 0.f;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a = fmaf(q[e], to_float<T>(t.e[e]), a);
+                sc[p] = a;
+            }
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
+        if (p < passes) {
+            // all lanes take part in the group reduction; dead slots carry -inf from one lane only
+            float a = sc[p] == -INFINITY ? 0.f : sc[p];
+            a = group_sum(a, LPS);
+            sc[p] = sc[p] == -INFINITY ? -INFINITY : a;
+            mx = fmaxf(mx, sc[p]);
+        }
+    }
+    for (int o = LPS; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float den = 0.f;
+#pragma unroll
+    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
+        if (p < passes) {
+            sc[p] = sc[p] == -INFINITY ? 0.f : expf(sc[p] - mx);
+            den += sc[p];
+        }
+    }
+    for (int o = LPS; o < 64; o <<= 1) den += __shfl_xor(den, o, 64);
+    den = fmaxf(den, 1.0e-5f);
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    float *wp = W ? W + (((size_t)b * N + n) * H + h) * S : nullptr;
+#pragma unroll
+    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
+        if (p < passes) {
+            const int t = p * SPW + sub;
+            const float w = sc[p] / den;
+            if (wp && gl == 0 && t < S) wp[t] = w;
+            const int r = slot_row(t);
+            if (r >= 0) {
+                Pk x = *reinterpret_cast<const Pk *>(vb + (size_t)r * rs);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, to_float<T>(x.e[e]), acc[e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        for (int o = LPS; o < 64; o <<= 1) acc[e] += __shfl_xor(acc[e], o, 64);
+    if (sub == 0) {
+        Pk o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.e[e] = from_float<T>(acc[e]);
+        *reinterpret_cast<Pk *>(Out + (((size_t)b * N + n) * H + h) * D + gl * VEC) = o;
+    }
+}
+
+template <typename T, int LPS>
+static int attn_gather_vec_launch(const void *q, const void *k, const void *v, const int32_t *idx,
+                                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
+                                  int L, int R, int causal, hipStream_t st) {
+    using S = typename T::storage;
+    constexpr int VEC = 16 / (int)sizeof(S);
+    const long units = (long)B * N * H;
+    const long blocks = (units + 3) / 4;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    const float scale = 1.0f / sqrtf((float)(VEC * LPS));
+    attn_gather_vec_kernel<T, VEC, LPS><<<(unsigned)blocks, 256, 0, st>>>(
+        (const S *)q, (const S *)k, (const S *)v, idx, mask, (S *)out, weights, B, N, M, H, L, R, causal, scale);
+    return check_launch("attn_gather_vec_kernel");
+}
+
+// returns HSA_ERR_UNSUPPORTED when the shape does not fit (the scalar kernel then runs)
+template <typename T>
+static int attn_gather_vec_try(const void *q, const void *k, const void *v, const int32_t *idx, const uint8_t *mask,
+                               void *out, float *weights, int B, int N, int M, int H, int D, int L, int R,
+                               int causal, hipStream_t st) {
+    constexpr int VEC = 16 / (int)sizeof(typename T::storage);
+    if (D % VEC != 0) return HSA_ERR_UNSUPPORTED;
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0) return HSA_ERR_UNSUPPORTED;
+    const int lps = D / VEC;
+    const int S = 2 * R + 1 + L;
+#define HSA_GV(LPSN)                                                                                         \
+    case LPSN:                                                                                               \
+        if ((S + 64 / LPSN - 1) / (64 / LPSN) > GATHER_MAX_PASSES) return HSA_ERR_UNSUPPORTED;               \
+        return attn_gather_vec_launch<T, LPSN>(q, k, v, idx, mask, out, weights, B, N, M, H, L, R, causal, st)
+    switch (lps) {
+        HSA_GV(2);
+        HSA_GV(4);
+        HSA_GV(8);
+        HSA_GV(16);
+        HSA_GV(32);
+    }
+#undef HSA_GV
+    return HSA_ERR_UNSUPPORTED;
+}
+
 template <typename T>
 int attn_gather_launch(const void *q, const void *k, const void *v, const int32_t *idx,
                        const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
@@ -142,6 +301,13 @@ int attn_gather_dispatch(const void *q, const void *k, const void *v, const int3
     if (2 * R + 1 + L > 64 * GATHER_MAX_CHUNKS)
         return fail(HSA_ERR_UNSUPPORTED, "2R+1+L = %d slots exceeds %d", 2 * R + 1 + L,
                     64 * GATHER_MAX_CHUNKS);
+    {
+        int rc = HSA_ERR_UNSUPPORTED;
+        if (dtype == HSA_F32) rc = attn_gather_vec_try<F32>(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, st);
+        else if (dtype == HSA_F16) rc = attn_gather_vec_try<F16>(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, st);
+        else if (dtype == HSA_BF16) rc = attn_gather_vec_try<BF16>(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, st);
+        if (rc != HSA_ERR_UNSUPPORTED) return rc;
+    }
     switch (dtype) {
         case HSA_F32: return attn_gather_launch<F32>(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, st);
         case HSA_F16: return attn_gather_launch<F16>(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, st);

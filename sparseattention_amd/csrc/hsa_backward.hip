@@ -329,11 +329,241 @@ attn_bwd_key_kernel(const typename T::storage *__restrict__ Q, const typename T:
     }
 }
 
+// ---- vector variants of the two passes (D a multiple of 16 bytes of elements) ----------------
+// Same lane mapping as the vector forward gather kernel: D/VEC lanes share a row and read it as
+// one contiguous piece.  Pass 1: a wavefront owns one query, 64*VEC/D slots per pass.  Pass 2: a
+// wavefront owns 64*VEC/D consecutive key rows, each lane group walks the queries of its row.
+constexpr int BWD_MAX_PASSES = 40;
+
+template <typename T, int VEC, int LPS>
+__global__ void __launch_bounds__(256)
+attn_bwd_query_vec_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ K,
+                          const typename T::storage *__restrict__ V, const typename T::storage *__restrict__ dO,
+                          typename T::storage *__restrict__ dQ, float *__restrict__ Pw, float *__restrict__ DS,
+                          int B, int N, int M, int H, int L, int R, int causal, float scale) {
+    constexpr int D = VEC * LPS;
+    constexpr int SPW = 64 / LPS;
+    struct alignas(16) Pk { typename T::storage e[VEC]; };
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPS, gl = lane % LPS;
+    const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= (long)B * N * H) return;
+    const int h = (int)(unit % H);
+    const int n = (int)((unit / H) % N);
+    const int b = (int)(unit / ((long)H * N));
+    const int Wn = 2 * R + 1, S = Wn + L;
+    const int passes = (S + SPW - 1) / SPW;
+    const size_t rs = (size_t)H * D;
+    const typename T::storage *kb = K + (size_t)b * M * rs + (size_t)h * D + gl * VEC;
+    const typename T::storage *vb = V + (size_t)b * M * rs + (size_t)h * D + gl * VEC;
+    const size_t qoff = (((size_t)b * N + n) * H + h) * D + gl * VEC;
+    float q[VEC], g[VEC];
+    {
+        Pk a = *reinterpret_cast<const Pk *>(Q + qoff), c = *reinterpret_cast<const Pk *>(dO + qoff);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { q[e] = to_float<T>(a.e[e]) * scale; g[e] = to_float<T>(c.e[e]); }
+    }
+    auto slot_row = [&](int t) {
+        int r = -1;
+        if (t < Wn) {
+            const int j = n + t - R;
+            if (j >= 0 && j < N && (!causal || j <= n)) r = j;
+        } else if (t < S) {
+            const int l = t - Wn;
+            if (!(causal && (((n >> l) & 1) == 0))) r = level_offset(N, l) + ((n >> l) ^ 1);
+        }
+        return r;
+    };
+    float sc[BWD_MAX_PASSES], dp[BWD_MAX_PASSES];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int p = 0; p < BWD_MAX_PASSES; ++p) {
+        sc[p] = -INFINITY;
+        dp[p] = 0.f;
+        if (p < passes) {
+            const int r = slot_row(p * SPW + sub);
+            float a = 0.f, c = 0.f;
+            if (r >= 0) {
+                Pk kk = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
+                Pk vv = *reinterpret_cast<const Pk *>(vb + (size_t)r * rs);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    a = fmaf(q[e], to_float<T>(kk.e[e]), a);
+                    c = fmaf(g[e], to_float<T>(vv.e[e]), c);
+                }
+            }
+            a = group_sum(a, LPS);
+            c = group_sum(c, LPS);
+            if (r >= 0) { sc[p] = a; dp[p] = c; }
+            mx = fmaxf(mx, sc[p]);
+        }
+    }
+    for (int o = LPS; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float den = 0.f;
+#pragma unroll
+    for (int p = 0; p < BWD_MAX_PASSES; ++p)
+        if (p < passes) { sc[p] = sc[p] == -INFINITY ? 0.f : expf(sc[p] - mx); den += sc[p]; }
+    for (int o = LPS; o < 64; o <<= 1) den += __shfl_xor(den, o, 64);
+    den = fmaxf(den, 1.0e-5f);
+    float dot = 0.f;
+#pragma unroll
+    for (int p = 0; p < BWD_MAX_PASSES; ++p)
+        if (p < passes) { sc[p] /= den; dot += sc[p] * dp[p]; }
+    for (int o = LPS; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
+    float *pw = Pw + (((size_t)b * N + n) * H + h) * S;
+    float *ds = DS + (((size_t)b * N + n) * H + h) * S;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int p = 0; p < BWD_MAX_PASSES; ++p) {
+        if (p < passes) {
+            const int t = p * SPW + sub;
+            const float s = sc[p] * (dp[p] - dot) * scale;
+            if (gl == 0 && t < S) { pw[t] = sc[p]; ds[t] = s; }
+            const int r = slot_row(t);
+            if (r >= 0) {
+                Pk kk = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(s, to_float<T>(kk.e[e]), acc[e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e)
+        for (int o = LPS; o < 64; o <<= 1) acc[e] += __shfl_xor(acc[e], o, 64);
+    if (sub == 0) {
+        Pk o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o.e[e] = from_float<T>(acc[e]);
+        *reinterpret_cast<Pk *>(dQ + qoff) = o;
+    }
+}
+
+template <typename T, int VEC, int LPS>
+__global__ void __launch_bounds__(256)
+attn_bwd_key_vec_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ dO,
+                        const float *__restrict__ Pw, const float *__restrict__ DS,
+                        typename T::storage *__restrict__ dK, typename T::storage *__restrict__ dV, int B, int N,
+                        int M, int H, int L, int R, int causal) {
+    constexpr int D = VEC * LPS;
+    constexpr int SPW = 64 / LPS;
+    struct alignas(16) Pk { typename T::storage e[VEC]; };
+    const int lane = threadIdx.x & 63;
+    const int sub = lane / LPS, gl = lane % LPS;
+    // unit = (batch, row group, head): SPW consecutive rows of one head per wavefront
+    const int groups = (M + SPW - 1) / SPW;
+    const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= (long)B * groups * H) return;
+    const int h = (int)(unit % H);
+    const int grp = (int)((unit / H) % groups);
+    const int b = (int)(unit / ((long)H * groups));
+    const int row = grp * SPW + sub;
+    if (row >= M) return;
+    const int Wn = 2 * R + 1, S = Wn + L;
+    const size_t rs = (size_t)H * D;
+    const typename T::storage *qb = Q + (size_t)b * N * rs + (size_t)h * D + gl * VEC;
+    const typename T::storage *gb = dO + (size_t)b * N * rs + (size_t)h * D + gl * VEC;
+    const float *pw = Pw + (size_t)b * N * H * S + (size_t)h * S;
+    const float *ds = DS + (size_t)b * N * H * S + (size_t)h * S;
+    const size_t ws = (size_t)H * S;
+    float ak[VEC], av[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) { ak[e] = 0.f; av[e] = 0.f; }
+    auto add = [&](int n, int slot) {
+        const float w = pw[(size_t)n * ws + slot];
+        const float s = ds[(size_t)n * ws + slot];
+        Pk qq = *reinterpret_cast<const Pk *>(qb + (size_t)n * rs);
+        Pk gg = *reinterpret_cast<const Pk *>(gb + (size_t)n * rs);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            ak[e] = fmaf(s, to_float<T>(qq.e[e]), ak[e]);
+            av[e] = fmaf(w, to_float<T>(gg.e[e]), av[e]);
+        }
+    };
+    if (row < N) {
+        const int lo = causal ? row : (row - R < 0 ? 0 : row - R);
+        const int hi = row + R >= N ? N - 1 : row + R;
+        for (int n = lo; n <= hi; ++n) add(n, row - n + R);
+        if (L > 0) {
+            const int sib = row ^ 1;
+            if (!causal || (sib & 1)) add(sib, Wn);
+        }
+    } else if (row < 2 * N - 2) {
+        int lvl = 1;
+        while (row >= level_offset(N, lvl + 1)) ++lvl;
+        const int pidx = row - level_offset(N, lvl);
+        if (!causal || (pidx & 1) == 0) {
+            const int first = (pidx ^ 1) << lvl;
+            for (int n = first; n < first + (1 << lvl); ++n) add(n, Wn + lvl);
+        }
+    }
+    Pk ok, ov;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) { ok.e[e] = from_float<T>(ak[e]); ov.e[e] = from_float<T>(av[e]); }
+    const size_t off = (((size_t)b * M + row) * H + h) * D + gl * VEC;
+    *reinterpret_cast<Pk *>(dK + off) = ok;
+    *reinterpret_cast<Pk *>(dV + off) = ov;
+}
+
+template <typename T, int LPS>
+static int attn_bwd_vec_launch(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                               void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int L, int R,
+                               int causal, hipStream_t st) {
+    using S = typename T::storage;
+    constexpr int VEC = 16 / (int)sizeof(S);
+    constexpr int SPW = 64 / LPS;
+    const float scale = 1.0f / sqrtf((float)(VEC * LPS));
+    long units = (long)B * N * H;
+    long blocks = (units + 3) / 4;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    attn_bwd_query_vec_kernel<T, VEC, LPS><<<(unsigned)blocks, 256, 0, st>>>(
+        (const S *)q, (const S *)k, (const S *)v, (const S *)dout, (S *)dq, ws_p, ws_ds, B, N, M, H, L, R, causal,
+        scale);
+    int rc = check_launch("attn_bwd_query_vec_kernel");
+    if (rc != HSA_OK) return rc;
+    units = (long)B * ((M + SPW - 1) / SPW) * H;
+    blocks = (units + 3) / 4;
+    if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    attn_bwd_key_vec_kernel<T, VEC, LPS><<<(unsigned)blocks, 256, 0, st>>>(
+        (const S *)q, (const S *)dout, ws_p, ws_ds, (S *)dk, (S *)dv, B, N, M, H, L, R, causal);
+    return check_launch("attn_bwd_key_vec_kernel");
+}
+
+template <typename T>
+static int attn_bwd_vec_try(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                            void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
+                            int causal, hipStream_t st) {
+    constexpr int VEC = 16 / (int)sizeof(typename T::storage);
+    if (D % VEC != 0) return HSA_ERR_UNSUPPORTED;
+    const uintptr_t al = (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dout | (uintptr_t)dq |
+                         (uintptr_t)dk | (uintptr_t)dv;
+    if ((al & 15) != 0) return HSA_ERR_UNSUPPORTED;
+    const int S = 2 * R + 1 + L;
+#define HSA_BV(LPSN)                                                                                          \
+    case LPSN:                                                                                                \
+        if ((S + 64 / LPSN - 1) / (64 / LPSN) > BWD_MAX_PASSES) return HSA_ERR_UNSUPPORTED;                   \
+        return attn_bwd_vec_launch<T, LPSN>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, L, R, causal, st)
+    switch (D / VEC) {
+        HSA_BV(2);
+        HSA_BV(4);
+        HSA_BV(8);
+        HSA_BV(16);
+        HSA_BV(32);
+    }
+#undef HSA_BV
+    return HSA_ERR_UNSUPPORTED;
+}
+
 template <typename T>
 static int attn_bwd_typed(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
                           void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
                           int causal, hipStream_t st) {
     using S = typename T::storage;
+    {
+        int rc = attn_bwd_vec_try<T>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal, st);
+        if (rc != HSA_ERR_UNSUPPORTED) return rc;
+    }
     const float scale = 1.0f / sqrtf((float)D);
     long units = (long)B * N * H;
     long blocks = (units + 3) / 4;
