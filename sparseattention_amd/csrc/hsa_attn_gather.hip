@@ -172,38 +172,40 @@ attn_gather_vec_kernel(const typename T::storage *__restrict__ Q, const typename
         }
         return r;
     };
-    // pass 1: scores of this lane group's slots (kept in registers, GATHER_MAX_PASSES bound)
+    // pass 1: scores of this lane group's slots, eight passes at a time: the eight key pieces are
+    // requested together and unconditionally (a dead slot re-reads the query's own leaf row, which
+    // is hot), so one memory round trip serves eight passes
+    constexpr int CHUNK = 8;
     float sc[GATHER_MAX_PASSES];
     float mx = -INFINITY;
 #pragma unroll
-    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
-        sc[p] = -INFINITY;
-        if (p < passes) {
-            const int r = slot_row(p * SPW + sub);
-            if (r >= 0) {
-                Pk t = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
+    for (int c = 0; c < GATHER_MAX_PASSES / CHUNK; ++c) {
+#pragma unroll
+        for (int p = 0; p < CHUNK; ++p) sc[c * CHUNK + p] = -INFINITY;
+        if (c * CHUNK < passes) {  // uniform
+            int rr[CHUNK];
+            Pk kk[CHUNK];
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
+                rr[p] = slot_row((c * CHUNK + p) * SPW + sub);
+                kk[p] = *reinterpret_cast<const Pk *>(kb + (size_t)(rr[p] < 0 ? n : rr[p]) * rs);
+            }
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
                 float a = 0.f;
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) a = fmaf(q[e], to_float<T>(t.e[e]), a);
-                sc[p] = a;
+                for (int e = 0; e < VEC; ++e) a = fmaf(q[e], to_float<T>(kk[p].e[e]), a);
+                a = group_sum(a, LPS);
+                if (rr[p] >= 0) sc[c * CHUNK + p] = a;
+                mx = fmaxf(mx, sc[c * CHUNK + p]);
             }
-        }
-    }
-#pragma unroll
-    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
-        if (p < passes) {
-            // all lanes take part in the group reduction; dead slots carry -inf from one lane only
-            float a = sc[p] == -INFINITY ? 0.f : sc[p];
-            a = group_sum(a, LPS);
-            sc[p] = sc[p] == -INFINITY ? -INFINITY : a;
-            mx = fmaxf(mx, sc[p]);
         }
     }
     for (int o = LPS; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
     float den = 0.f;
 #pragma unroll
     for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
-        if (p < passes) {
+        if ((p / CHUNK) * CHUNK < passes) {  // every pass of an active chunk (dead slots become 0)
             sc[p] = sc[p] == -INFINITY ? 0.f : expf(sc[p] - mx);
             den += sc[p];
         }
@@ -215,16 +217,22 @@ attn_gather_vec_kernel(const typename T::storage *__restrict__ Q, const typename
     for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
     float *wp = W ? W + (((size_t)b * N + n) * H + h) * S : nullptr;
 #pragma unroll
-    for (int p = 0; p < GATHER_MAX_PASSES; ++p) {
-        if (p < passes) {
-            const int t = p * SPW + sub;
-            const float w = sc[p] / den;
-            if (wp && gl == 0 && t < S) wp[t] = w;
-            const int r = slot_row(t);
-            if (r >= 0) {
-                Pk x = *reinterpret_cast<const Pk *>(vb + (size_t)r * rs);
+    for (int c = 0; c < GATHER_MAX_PASSES / CHUNK; ++c) {
+        if (c * CHUNK < passes) {  // uniform
+            int rr[CHUNK];
+            Pk vv[CHUNK];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, to_float<T>(x.e[e]), acc[e]);
+            for (int p = 0; p < CHUNK; ++p) {
+                rr[p] = slot_row((c * CHUNK + p) * SPW + sub);
+                vv[p] = *reinterpret_cast<const Pk *>(vb + (size_t)(rr[p] < 0 ? n : rr[p]) * rs);
+            }
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
+                const int t = (c * CHUNK + p) * SPW + sub;
+                const float w = sc[c * CHUNK + p] / den;  // zero for dead slots
+                if (wp && gl == 0 && t < S) wp[t] = w;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, to_float<T>(vv[p].e[e]), acc[e]);
             }
         }
     }

@@ -374,41 +374,51 @@ attn_bwd_query_vec_kernel(const typename T::storage *__restrict__ Q, const typen
         }
         return r;
     };
+    // eight passes at a time: key and value pieces requested together and unconditionally
+    // (a dead slot re-reads the query's own leaf row)
+    constexpr int CHUNK = 8;
     float sc[BWD_MAX_PASSES], dp[BWD_MAX_PASSES];
     float mx = -INFINITY;
 #pragma unroll
-    for (int p = 0; p < BWD_MAX_PASSES; ++p) {
-        sc[p] = -INFINITY;
-        dp[p] = 0.f;
-        if (p < passes) {
-            const int r = slot_row(p * SPW + sub);
-            float a = 0.f, c = 0.f;
-            if (r >= 0) {
-                Pk kk = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
-                Pk vv = *reinterpret_cast<const Pk *>(vb + (size_t)r * rs);
+    for (int c = 0; c < BWD_MAX_PASSES / CHUNK; ++c) {
+#pragma unroll
+        for (int p = 0; p < CHUNK; ++p) { sc[c * CHUNK + p] = -INFINITY; dp[c * CHUNK + p] = 0.f; }
+        if (c * CHUNK < passes) {  // uniform
+            int rr[CHUNK];
+            Pk kk[CHUNK], vv[CHUNK];
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
+                rr[p] = slot_row((c * CHUNK + p) * SPW + sub);
+                const size_t ro = (size_t)(rr[p] < 0 ? n : rr[p]) * rs;
+                kk[p] = *reinterpret_cast<const Pk *>(kb + ro);
+                vv[p] = *reinterpret_cast<const Pk *>(vb + ro);
+            }
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
+                float a = 0.f, cc = 0.f;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    a = fmaf(q[e], to_float<T>(kk.e[e]), a);
-                    c = fmaf(g[e], to_float<T>(vv.e[e]), c);
+                    a = fmaf(q[e], to_float<T>(kk[p].e[e]), a);
+                    cc = fmaf(g[e], to_float<T>(vv[p].e[e]), cc);
                 }
+                a = group_sum(a, LPS);
+                cc = group_sum(cc, LPS);
+                if (rr[p] >= 0) { sc[c * CHUNK + p] = a; dp[c * CHUNK + p] = cc; }
+                mx = fmaxf(mx, sc[c * CHUNK + p]);
             }
-            a = group_sum(a, LPS);
-            c = group_sum(c, LPS);
-            if (r >= 0) { sc[p] = a; dp[p] = c; }
-            mx = fmaxf(mx, sc[p]);
         }
     }
     for (int o = LPS; o < 64; o <<= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
     float den = 0.f;
 #pragma unroll
     for (int p = 0; p < BWD_MAX_PASSES; ++p)
-        if (p < passes) { sc[p] = sc[p] == -INFINITY ? 0.f : expf(sc[p] - mx); den += sc[p]; }
+        if ((p / CHUNK) * CHUNK < passes) { sc[p] = sc[p] == -INFINITY ? 0.f : expf(sc[p] - mx); den += sc[p]; }
     for (int o = LPS; o < 64; o <<= 1) den += __shfl_xor(den, o, 64);
     den = fmaxf(den, 1.0e-5f);
     float dot = 0.f;
 #pragma unroll
     for (int p = 0; p < BWD_MAX_PASSES; ++p)
-        if (p < passes) { sc[p] /= den; dot += sc[p] * dp[p]; }
+        if ((p / CHUNK) * CHUNK < passes) { sc[p] /= den; dot += sc[p] * dp[p]; }
     for (int o = LPS; o < 64; o <<= 1) dot += __shfl_xor(dot, o, 64);
     float *pw = Pw + (((size_t)b * N + n) * H + h) * S;
     float *ds = DS + (((size_t)b * N + n) * H + h) * S;
@@ -416,16 +426,21 @@ attn_bwd_query_vec_kernel(const typename T::storage *__restrict__ Q, const typen
 #pragma unroll
     for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
 #pragma unroll
-    for (int p = 0; p < BWD_MAX_PASSES; ++p) {
-        if (p < passes) {
-            const int t = p * SPW + sub;
-            const float s = sc[p] * (dp[p] - dot) * scale;
-            if (gl == 0 && t < S) { pw[t] = sc[p]; ds[t] = s; }
-            const int r = slot_row(t);
-            if (r >= 0) {
-                Pk kk = *reinterpret_cast<const Pk *>(kb + (size_t)r * rs);
+    for (int c = 0; c < BWD_MAX_PASSES / CHUNK; ++c) {
+        if (c * CHUNK < passes) {  // uniform
+            Pk kk[CHUNK];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(s, to_float<T>(kk.e[e]), acc[e]);
+            for (int p = 0; p < CHUNK; ++p) {
+                const int r = slot_row((c * CHUNK + p) * SPW + sub);
+                kk[p] = *reinterpret_cast<const Pk *>(kb + (size_t)(r < 0 ? n : r) * rs);
+            }
+#pragma unroll
+            for (int p = 0; p < CHUNK; ++p) {
+                const int t = (c * CHUNK + p) * SPW + sub;
+                const float s = sc[c * CHUNK + p] * (dp[c * CHUNK + p] - dot) * scale;  // zero for dead slots
+                if (gl == 0 && t < S) { pw[t] = sc[c * CHUNK + p]; ds[t] = s; }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) acc[e] = fmaf(s, to_float<T>(kk[p].e[e]), acc[e]);
             }
         }
     }
@@ -484,6 +499,7 @@ attn_bwd_key_vec_kernel(const typename T::storage *__restrict__ Q, const typenam
     if (row < N) {
         const int lo = causal ? row : (row - R < 0 ? 0 : row - R);
         const int hi = row + R >= N ? N - 1 : row + R;
+#pragma unroll 4
         for (int n = lo; n <= hi; ++n) add(n, row - n + R);
         if (L > 0) {
             const int sib = row ^ 1;
@@ -495,6 +511,7 @@ attn_bwd_key_vec_kernel(const typename T::storage *__restrict__ Q, const typenam
         const int pidx = row - level_offset(N, lvl);
         if (!causal || (pidx & 1) == 0) {
             const int first = (pidx ^ 1) << lvl;
+#pragma unroll 4
             for (int n = first; n < first + (1 << lvl); ++n) add(n, Wn + lvl);
         }
     }
