@@ -151,11 +151,16 @@ int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, cons
  * weights and writes dQ plus the weights / dS workspaces, the per-key pass gathers dK and dV
  * (fp32 accumulation, written once in the element type; rows that nobody attends get zeros).
  *   q, dout, dq  [B, N, H, D];  k, v, dk, dv  [B, M, H, D], M >= 2N-1
- *   ws_p, ws_ds  device float [B, N, H, 2R+1+L] each (workspace provided by the caller)
+ *   workspace    device memory of at least hsa_attn_bwd_workspace_bytes(...) bytes, provided by
+ *                the caller (scratch only: nothing in it has to survive the call)
+ *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit, head_dim 64, R <= 32:
+ *                fp32 atomics for tree levels >= 4), else the deterministic gather kernels
  */
+#include <stddef.h>
+size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo);
 int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
-                 void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
-                 int causal, int dtype, void *stream);
+                 void *dv, void *workspace, size_t workspace_bytes, int B, int N, int M, int H, int D,
+                 int L, int R, int causal, int dtype, int algo, void *stream);
 
 /*
  * Backward of the initial span nodes (the reference differentiates generate_span_input_Y,

@@ -46,7 +46,9 @@ def _declare(lib):
     lib.hsa_span_input_y.restype = I
     lib.hsa_build_parents_bwd.argtypes = [P] * 11 + [I] * 5 + [P]
     lib.hsa_build_parents_bwd.restype = I
-    lib.hsa_attn_bwd.argtypes = [P] * 9 + [I] * 9 + [P]
+    lib.hsa_attn_bwd_workspace_bytes.argtypes = [I] * 9
+    lib.hsa_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.hsa_attn_bwd.argtypes = [P] * 8 + [ctypes.c_size_t] + [I] * 10 + [P]
     lib.hsa_attn_bwd.restype = I
     lib.hsa_span_input_y_bwd.argtypes = [P, P, I, I, I, I, P]
     lib.hsa_span_input_y_bwd.restype = I

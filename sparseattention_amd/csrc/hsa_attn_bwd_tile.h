@@ -1,0 +1,519 @@
+// Span attention backward, MFMA tile kernels (16-bit element types, canonical tree tables).
+//
+// Two launches, the flash-attention split adapted to the window + tree structure:
+//
+//  (A) query-stationary, one wavefront per (batch, head, 16-query block): recomputes the score
+//      tiles S^T[key, query] exactly like the forward, then
+//          dP^T = V_blk . dO_blk^T          delta[q] = sum_key P dP
+//          dS^T = P (dP - delta) / sqrt(D)   dQ^T[ch, q] = K_blk^T . dS^T
+//      and stores dQ plus two numbers per (query, head): the log2-domain log-sum-exp and delta.
+//      The tree key blocks are also evaluated in the other orientation (S[query, slot]), which
+//      puts the queries into the MFMA contraction: dK^T[ch, slot] = Q^T . dS, dV^T = dO^T . P.
+//      Nodes of levels 1..3 are attended only from inside the block: their rows are final and
+//      written directly.  Nodes of levels >= 4 collect from 2^(l-4) blocks: fp32 atomic adds
+//      into a small accumulation buffer (N/8 rows per sequence), converted afterwards.
+//  (B) key-stationary, one wavefront per (batch, head, 16-leaf key block): loops over the query
+//      blocks whose window reaches the key block, rebuilds P and dS from the saved statistics
+//      and accumulates dK^T = Q^T . dS, dV^T = dO^T . P in registers.  Every leaf row of dK / dV
+//      is written once; no atomics.
+//
+// Operand plumbing is the forward kernel's: row-contiguous 16-byte global accesses, per-wavefront
+// LDS re-layout into MFMA operand order, transposed operands through an MFMA with a 0/1
+// selection matrix.
+#pragma once
+
+#include "hsa_attn_tile.h"
+
+namespace hsa {
+
+struct BwdTileParams {
+    const uint16_t *q, *k, *v, *dout;
+    uint16_t *dq, *dk, *dv;
+    float *stats;   // [B, N, H, 2]: log2-domain lse, delta
+    float *upper;   // [2, B, NU, H, D] fp32 accumulators of dK, dV rows of tree levels >= 4
+    int B, N, M, H, L, R;
+    int NU;         // rows of levels >= 4: (2N-1) - off_4 (0 when L < 5)
+    int n_units;
+    float scale_log2e, scale;
+};
+
+constexpr int BWD_WPB = 4;  // wavefronts per workgroup
+
+template <typename T, int D>
+struct BwdTile {
+    using M_ = Mma<T>;
+    static constexpr int KS = D / 32, NJ = D / 16, CPR = D / 8, RPI = 64 / CPR, NLD = TILE_Q / RPI;
+    static constexpr int PITCH = D * 2 + 16, BLK_BYTES = TILE_Q * PITCH;
+
+    int lane, r16, g, lrow, lchk;
+    unsigned char *lds;
+    u32x4_t Pi[2];
+
+    __device__ __forceinline__ void init(unsigned char *wave_lds) {
+        lane = threadIdx.x & 63;
+        r16 = lane & 15;
+        g = lane >> 4;
+        lrow = lane / CPR;
+        lchk = lane % CPR;
+        lds = wave_lds;
+#pragma unroll
+        for (int jj = 0; jj < 2; ++jj) {
+            const int e = 4 * jj + (r16 & 3);
+            const uint32_t one = (g == (r16 >> 2)) ? (uint32_t)M_::kOne << (16 * (e & 1)) : 0u;
+            const int wi = e >> 1;
+            Pi[jj] = u32x4_t{wi == 0 ? one : 0u, wi == 1 ? one : 0u, wi == 2 ? one : 0u, wi == 3 ? one : 0u};
+        }
+    }
+    // rows -> LDS -> operand pieces
+    __device__ __forceinline__ void put(int slot, const u32x4_t (&raw)[NLD]) const {
+        unsigned char *reg = lds + slot * BLK_BYTES + lrow * PITCH + 16 * lchk;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) *reinterpret_cast<u32x4_t *>(reg + i * RPI * PITCH) = raw[i];
+    }
+    __device__ __forceinline__ void get(int slot, u32x4_t (&dst)[KS]) const {
+        const unsigned char *reg = lds + slot * BLK_BYTES + r16 * PITCH + 16 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const u32x4_t *>(reg + 64 * ks);
+    }
+    // operand rows -> "lane = channel, regs = rows" form
+    __device__ __forceinline__ void transpose(const u32x4_t (&op)[KS], u32x2_t (&dst)[NJ]) const {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            f32x4 r = M_::k32(op[j >> 1], Pi[j & 1], z);
+            dst[j] = u32x2_t{M_::pack_exact(r[0], r[1]), M_::pack_exact(r[2], r[3])};
+        }
+    }
+    // result tiles [channel, column] (this lane: column r16, channels 32ks+8g+4jj+i) -> packed
+    // 16-bit pieces in LDS slot `slot`, one row per column
+    __device__ __forceinline__ void put_result(int slot, const f32x4 (&t)[NJ], float mul) const {
+        unsigned char *reg = lds + slot * BLK_BYTES + r16 * PITCH + 16 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const f32x4 a = t[2 * ks], b = t[2 * ks + 1];
+            *reinterpret_cast<u32x4_t *>(reg + 64 * ks) =
+                u32x4_t{M_::pack(a[0] * mul, a[1] * mul), M_::pack(a[2] * mul, a[3] * mul),
+                        M_::pack(b[0] * mul, b[1] * mul), M_::pack(b[2] * mul, b[3] * mul)};
+        }
+    }
+    __device__ __forceinline__ u32x4_t get_row_piece(int slot, int i) const {
+        return *reinterpret_cast<const u32x4_t *>(lds + slot * BLK_BYTES + (i * RPI + lrow) * PITCH + 16 * lchk);
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// (A) query-stationary pass
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D, int NBW, bool CAUSAL>
+__global__ void __launch_bounds__(BWD_WPB * 64)
+attn_bwd_tile_query_kernel(BwdTileParams p) {
+    using BT = BwdTile<T, D>;
+    using M_ = Mma<T>;
+    constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD;
+    constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
+    constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
+    constexpr int LDS_SLOTS = 4;
+    __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = blockIdx.x * BWD_WPB + wave;
+    if (unit >= p.n_units) return;
+    BT bt;
+    bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
+    const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
+
+    const int N = p.N, L = p.L, R = p.R, H = p.H;
+    const int NB = N / TILE_Q;
+    const int h = unit % H;
+    const int blk = (unit / H) % NB;
+    const int b = unit / (H * NB);
+    const int q0 = blk * TILE_Q;
+    const size_t rs = (size_t)H * D;
+    const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Kb = p.k + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    const uint16_t *Vb = p.v + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+
+    // ---- tree slot constants (same slot layout as the forward kernel) -------------------------
+    int t_row[NLD], u_row[NLD];     // rows this lane fetches / stores, -1 = slot does not exist
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int sl = i * RPI + lrow;
+        int lvl, add, x;
+        if (sl < 8) { lvl = 1; add = sl; x = 0; }
+        else if (sl < 12) { lvl = 2; add = sl - 8; x = 0; }
+        else if (sl < 14) { lvl = 3; add = sl - 12; x = 0; }
+        else { lvl = 4 + (sl - 14); add = 0; x = 1; }
+        t_row[i] = lvl < L ? level_offset(N, lvl) + (((q0 >> lvl) + add) ^ x) : -1;
+        const int ul = 6 + sl;
+        u_row[i] = ul < L ? level_offset(N, ul) + ((q0 >> ul) ^ 1) : -1;
+    }
+    auto slot_level = [](int sl, int &pl) {  // near slot -> level, position under the ancestor (-1: sibling slot)
+        if (sl < 8) { pl = sl; return 1; }
+        if (sl < 12) { pl = sl - 8; return 2; }
+        if (sl < 14) { pl = sl - 12; return 3; }
+        pl = -1;
+        return 4 + (sl - 14);
+    };
+    // orientation 1 (lane = query r16, regs = slots 4g+i) and orientation 2 (lane = slot r16,
+    // regs = queries 4g+i) liveness of the near and far blocks
+    float b1T[4], b1U[4], b2T[4], b2U[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        {
+            int pl;
+            const int lvl = slot_level(4 * g + i, pl);
+            bool live = pl >= 0 ? (pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1)))
+                                : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+            b1T[i] = live ? 0.f : NEG_INF;
+            const int ul = 6 + 4 * g + i;
+            b1U[i] = (ul < L && (!CAUSAL || ((q0 >> ul) & 1))) ? 0.f : NEG_INF;
+        }
+        {
+            int pl;
+            const int lvl = slot_level(r16, pl);
+            const int ql = 4 * g + i;
+            bool live = pl >= 0 ? (pl == ((ql >> lvl) ^ 1) && (!CAUSAL || ((ql >> lvl) & 1)))
+                                : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+            b2T[i] = live ? 0.f : NEG_INF;
+            const int ul = 6 + r16;
+            b2U[i] = (ul < L && (!CAUSAL || ((q0 >> ul) & 1))) ? 0.f : NEG_INF;
+        }
+    }
+    float biasL[NKL][4];
+#pragma unroll
+    for (int c = 0; c < NKL; ++c) {
+        const int dlt = TILE_Q * (c - NBW);
+        const int kb = blk - NBW + c;
+        const bool inside = kb >= 0 && kb < NB;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kl = 4 * g + i;
+            const int diff = dlt + kl - r16;
+            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+            const bool sib = dlt == 0 && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
+            const int cnt = (int)win + (int)sib;
+            biasL[c][i] = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+        }
+    }
+
+    // ---- loads ------------------------------------------------------------------------------
+    auto load_block = [&](const uint16_t *base, int row0, u32x4_t (&dst)[NLD]) {
+        const uint16_t *ptr = base + (size_t)(row0 + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) dst[i] = *reinterpret_cast<const u32x4_t *>(ptr + (size_t)(i * RPI) * rs);
+    };
+    auto load_rows = [&](const uint16_t *base, const int (&rows)[NLD], u32x4_t (&dst)[NLD]) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            dst[i] = *reinterpret_cast<const u32x4_t *>(base + (size_t)(rows[i] < 0 ? q0 : rows[i]) * rs);
+    };
+    u32x4_t rQ[NLD], rG[NLD], rK[NKB][NLD], rV[NKB][NLD];
+    load_block(Qb, q0, rQ);
+    load_block(Gb, q0, rG);
+#pragma unroll
+    for (int c = 0; c < NKL; ++c) {
+        int kb = blk - NBW + c;
+        kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
+        load_block(Kb, kb * TILE_Q, rK[c]);
+        load_block(Vb, kb * TILE_Q, rV[c]);
+    }
+    load_rows(Kb, t_row, rK[NKL]);
+    load_rows(Vb, t_row, rV[NKL]);
+    load_rows(Kb, u_row, rK[NKL + 1]);
+    load_rows(Vb, u_row, rV[NKL + 1]);
+
+    // ---- operand forms ------------------------------------------------------------------------
+    u32x4_t Qf[KS], Gf[KS], Kc[NKB][KS], Vc[NKB][KS];
+    bt.put(0, rQ);
+    bt.put(1, rG);
+    bt.get(0, Qf);
+    bt.get(1, Gf);
+#pragma unroll
+    for (int c = 0; c < NKB; ++c) {
+        bt.put(2, rK[c]);
+        bt.put(3, rV[c]);
+        bt.get(2, Kc[c]);
+        bt.get(3, Vc[c]);
+    }
+
+    // ---- orientation 1: S^T, dP^T [key, query] ---------------------------------------------------
+    float sc[NKB][4], dp[NKB][4];
+    float mx = NEG_INF;
+#pragma unroll
+    for (int c = 0; c < NKB; ++c) {
+        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            a = M_::k32(Kc[c][ks], Qf[ks], a);
+            d = M_::k32(Vc[c][ks], Gf[ks], d);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
+            sc[c][i] = fmaf(a[i], p.scale_log2e, bias);
+            dp[c][i] = d[i];
+            mx = fmaxf(mx, sc[c][i]);
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float den = 0.f;
+#pragma unroll
+    for (int c = 0; c < NKB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sc[c][i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
+            den += sc[c][i];
+        }
+    den += __shfl_xor(den, 16, 64);
+    den += __shfl_xor(den, 32, 64);
+    const float inv = 1.0f / den;
+    float delta = 0.f;
+#pragma unroll
+    for (int c = 0; c < NKB; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            sc[c][i] *= inv;  // P
+            delta = fmaf(sc[c][i], dp[c][i], delta);
+        }
+    delta += __shfl_xor(delta, 16, 64);
+    delta += __shfl_xor(delta, 32, 64);
+    const float lse = mx + __builtin_amdgcn_logf(den);  // log2 domain: P = exp2(s' - lse)
+    if (g == 0) {
+        float *st = p.stats + (((size_t)b * N + q0 + r16) * H + h) * 2;
+        st[0] = lse;
+        st[1] = delta;
+    }
+
+    // ---- dQ^T = sum_c K_c^T . dS_c^T ---------------------------------------------------------------
+    {
+        f32x4 acc[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NKB; ++c) {
+            u32x2_t KT[NJ];
+            bt.transpose(Kc[c], KT);
+            float ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ds[i] = sc[c][i] * (dp[c][i] - delta) * p.scale;
+            const u32x2_t dsp = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) acc[j] = M_::k16(KT[j], dsp, acc[j]);
+        }
+        bt.put_result(0, acc, 1.0f);
+        uint16_t *optr = p.dq + ((size_t)b * N * H + h) * D + 8 * lchk + (size_t)(q0 + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
+    }
+
+    // ---- orientation 2 for the tree blocks: dK^T, dV^T [channel, slot] ------------------------------
+    u32x2_t QT[NJ], GT[NJ];
+    bt.transpose(Qf, QT);
+    bt.transpose(Gf, GT);
+    float lse4[4], del4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        lse4[i] = __shfl(lse, 4 * g + i, 64);
+        del4[i] = __shfl(delta, 4 * g + i, 64);
+    }
+    uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const int c = NKL + t;
+        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            a = M_::k32(Qf[ks], Kc[c][ks], a);   // S[query 4g+i, slot r16]
+            d = M_::k32(Gf[ks], Vc[c][ks], d);   // dP[query, slot]
+        }
+        float pp[4], ds[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float bias = t == 0 ? b2T[i] : b2U[i];
+            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
+            ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
+        }
+        const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+        const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+        f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            tk[j] = M_::k16(QT[j], dk, z);
+            tv[j] = M_::k16(GT[j], pk, z);
+        }
+        if (t == 0) {
+            // slots 0..13 (levels 1..3) are complete: rows written directly
+            bt.put_result(0, tk, 1.0f);
+            bt.put_result(1, tv, 1.0f);
+#pragma unroll
+            for (int i = 0; i < NLD; ++i) {
+                const int sl = i * RPI + lrow;
+                if (sl < 14 && t_row[i] >= 0) {
+                    *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
+                    *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
+                }
+            }
+        }
+        // slots of levels >= 4 accumulate over blocks: fp32 atomics
+        const int lvl = t == 0 ? (r16 >= 14 ? 4 + (r16 - 14) : -1) : 6 + r16;
+        if (lvl >= 4 && lvl < L) {
+            const int row = level_offset(N, lvl) + ((q0 >> lvl) ^ 1);
+            const size_t uo = (((size_t)b * p.NU + (row - level_offset(N, 4))) * H + h) * D;
+            float *uk = p.upper + uo;
+            float *uv = p.upper + (size_t)p.B * p.NU * H * D + uo;
+            const bool live = !CAUSAL || ((q0 >> lvl) & 1);
+            if (live) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1) + i;
+                        unsafeAtomicAdd(uk + ch, tk[j][i]);
+                        unsafeAtomicAdd(uv + ch, tv[j][i]);
+                    }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// (B) key-stationary pass over the leaf key blocks
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D, int NBW, bool CAUSAL>
+__global__ void __launch_bounds__(BWD_WPB * 64)
+attn_bwd_tile_key_kernel(BwdTileParams p) {
+    using BT = BwdTile<T, D>;
+    using M_ = Mma<T>;
+    constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD;
+    constexpr int NQB = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // query blocks that reach a key block
+    constexpr int LDS_SLOTS = 4;
+    __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = blockIdx.x * BWD_WPB + wave;
+    if (unit >= p.n_units) return;
+    BT bt;
+    bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
+    const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
+
+    const int N = p.N, R = p.R, H = p.H;
+    const int NB = N / TILE_Q;
+    const int h = unit % H;
+    const int kb = (unit / H) % NB;
+    const int b = unit / (H * NB);
+    const int k0 = kb * TILE_Q;
+    const size_t rs = (size_t)H * D;
+    const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Kb = p.k + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    const uint16_t *Vb = p.v + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+
+    auto load_block = [&](const uint16_t *base, int row0, u32x4_t (&dst)[NLD]) {
+        const uint16_t *ptr = base + (size_t)(row0 + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) dst[i] = *reinterpret_cast<const u32x4_t *>(ptr + (size_t)(i * RPI) * rs);
+    };
+    u32x4_t rK[NLD], rV[NLD], rQ[NQB][NLD], rG[NQB][NLD];
+    load_block(Kb, k0, rK);
+    load_block(Vb, k0, rV);
+    float lse4[NQB][4], del4[NQB][4];
+#pragma unroll
+    for (int c = 0; c < NQB; ++c) {
+        int qb = kb + (CAUSAL ? c : c - NBW);
+        qb = qb < 0 ? 0 : (qb >= NB ? NB - 1 : qb);
+        load_block(Qb, qb * TILE_Q, rQ[c]);
+        load_block(Gb, qb * TILE_Q, rG[c]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float *st = p.stats + (((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h) * 2;
+            lse4[c][i] = st[0];
+            del4[c][i] = st[1];
+        }
+    }
+    u32x4_t Kf[KS], Vf[KS];
+    bt.put(0, rK);
+    bt.put(1, rV);
+    bt.get(0, Kf);
+    bt.get(1, Vf);
+
+    f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+    for (int c = 0; c < NQB; ++c) {
+        const int qb = kb + (CAUSAL ? c : c - NBW);
+        const bool inside = qb >= 0 && qb < NB;  // uniform
+        u32x4_t Qf[KS], Gf[KS];
+        bt.put(2, rQ[c]);
+        bt.put(3, rG[c]);
+        bt.get(2, Qf);
+        bt.get(3, Gf);
+        u32x2_t QT[NJ], GT[NJ];
+        bt.transpose(Qf, QT);
+        bt.transpose(Gf, GT);
+        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            a = M_::k32(Qf[ks], Kf[ks], a);  // S[query 4g+i of block qb, key r16]
+            d = M_::k32(Gf[ks], Vf[ks], d);
+        }
+        float pp[4], ds[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ql = 4 * g + i;
+            const int diff = (kb - qb) * TILE_Q + r16 - ql;  // key - query
+            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+            const bool sib = qb == kb && r16 == (ql ^ 1) && (!CAUSAL || (ql & 1));
+            const int cnt = (int)win + (int)sib;
+            const float bias = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[c][i]);
+            ds[i] = pp[i] * (d[i] - del4[c][i]) * p.scale;
+        }
+        const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+        const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            tk[j] = M_::k16(QT[j], dk, tk[j]);
+            tv[j] = M_::k16(GT[j], pk, tv[j]);
+        }
+    }
+    bt.put_result(0, tk, 1.0f);
+    bt.put_result(1, tv, 1.0f);
+    uint16_t *dKp = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
+    uint16_t *dVp = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        *reinterpret_cast<u32x4_t *>(dKp + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
+        *reinterpret_cast<u32x4_t *>(dVp + (size_t)(i * RPI) * rs) = bt.get_row_piece(1, i);
+    }
+}
+
+// rows of tree levels >= 4: fp32 accumulators -> element type; the root and any extra rows get zeros
+template <typename T>
+__global__ void attn_bwd_tile_finish_kernel(const float *__restrict__ upper, uint16_t *__restrict__ dk,
+                                            uint16_t *__restrict__ dv, int B, int N, int M, int H, int D, int NU,
+                                            int first_upper_row) {
+    const size_t per_b = (size_t)(M - first_upper_row) * H * D;
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= (size_t)B * per_b) return;
+    const int b = (int)(t / per_b);
+    const size_t r = t % per_b;
+    const int row = first_upper_row + (int)(r / ((size_t)H * D));
+    const size_t hd = r % ((size_t)H * D);
+    float vk = 0.f, vv = 0.f;
+    if (row < 2 * N - 2) {  // below the root
+        const size_t uo = ((size_t)b * NU + (row - first_upper_row)) * H * D + hd;
+        vk = upper[uo];
+        vv = upper[(size_t)B * NU * H * D + uo];
+    }
+    const size_t o = ((size_t)b * M + row) * H * D + hd;
+    dk[o] = from_float<T>(vk);
+    dv[o] = from_float<T>(vv);
+}
+
+}  // namespace hsa

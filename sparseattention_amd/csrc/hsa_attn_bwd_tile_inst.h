@@ -1,0 +1,35 @@
+// Instantiates the tile backward kernels of one element type (head_dim 64).
+#pragma once
+#include "hsa_attn_bwd_tile.h"
+
+namespace hsa {
+
+template <typename T, int D, int NBW, bool CAUSAL>
+static int bwd_tile_launch_one(const BwdTileParams &p, hipStream_t st) {
+    const int nwg = (p.n_units + BWD_WPB - 1) / BWD_WPB;
+    attn_bwd_tile_query_kernel<T, D, NBW, CAUSAL><<<nwg, BWD_WPB * 64, 0, st>>>(p);
+    int rc = check_launch("attn_bwd_tile_query_kernel");
+    if (rc != HSA_OK) return rc;
+    attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL><<<nwg, BWD_WPB * 64, 0, st>>>(p);
+    return check_launch("attn_bwd_tile_key_kernel");
+}
+
+template <typename T, int D>
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, hipStream_t st);
+
+#define HSA_BWD_TILE_INSTANTIATE(T, D)                                                         \
+    template <>                                                                                \
+    int attn_bwd_tile_launch_td<T, D>(const BwdTileParams &p, int nbw, bool causal,            \
+                                      hipStream_t st) {                                        \
+        switch (nbw * 2 + (causal ? 1 : 0)) {                                                  \
+            case 0: return bwd_tile_launch_one<T, D, 0, false>(p, st);                         \
+            case 1: return bwd_tile_launch_one<T, D, 0, true>(p, st);                          \
+            case 2: return bwd_tile_launch_one<T, D, 1, false>(p, st);                         \
+            case 3: return bwd_tile_launch_one<T, D, 1, true>(p, st);                          \
+            case 4: return bwd_tile_launch_one<T, D, 2, false>(p, st);                         \
+            case 5: return bwd_tile_launch_one<T, D, 2, true>(p, st);                          \
+        }                                                                                      \
+        return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward");    \
+    }
+
+}  // namespace hsa

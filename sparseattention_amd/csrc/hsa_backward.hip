@@ -13,9 +13,12 @@
 //                     dK = sum dS Q, dV = sum P dO in fp32, written once in the element type.
 //                 Canonical complete-binary-tree tables only.
 //  span nodes     dx[n] = sum_l 2^-l dY[level l, n >> l].
-#include "hsa_common.h"
+#include "hsa_attn_bwd_tile.h"
 
 namespace hsa {
+
+template <typename T, int D>
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, hipStream_t st);
 
 // ---------------------------------------------------------------- parent build
 template <typename T, int VEC> struct BPack { typename T::storage e[VEC]; };
@@ -617,6 +620,62 @@ __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, ty
     dX[t] = from_float<T>(acc);
 }
 
+// ---------------------------------------------------------------- tile backward dispatch
+__global__ void bwd_zero_kernel(float *p, size_t n) {
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) p[t] = 0.f;
+}
+
+static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype) {
+    if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
+    if (D != 64) return false;
+    if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
+    if ((R + TILE_Q - 1) / TILE_Q > 2) return false;
+    return true;
+}
+
+static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
+    return 2 * (size_t)B * N * H * (2 * R + 1 + L);
+}
+static int bwd_tile_nu(int N, int L) { return L >= 4 ? (2 * N - 1) - level_offset(N, 4) : 0; }
+static size_t bwd_tile_ws_floats(int B, int N, int H, int D, int L) {
+    return (size_t)B * N * H * 2 + 2 * (size_t)B * bwd_tile_nu(N, L) * H * D;
+}
+
+template <typename T>
+static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                               void *dv, float *ws, int B, int N, int M, int H, int D, int L, int R, int causal,
+                               hipStream_t st) {
+    BwdTileParams p;
+    p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v; p.dout = (const uint16_t *)dout;
+    p.dq = (uint16_t *)dq; p.dk = (uint16_t *)dk; p.dv = (uint16_t *)dv;
+    p.stats = ws;
+    p.upper = ws + (size_t)B * N * H * 2;
+    p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
+    p.NU = bwd_tile_nu(N, L);
+    const long units = (long)B * (N / TILE_Q) * H;
+    if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.n_units = (int)units;
+    p.scale = 1.0f / sqrtf((float)D);
+    p.scale_log2e = 1.4426950408889634f * p.scale;
+    const size_t nup = 2 * (size_t)B * p.NU * H * D;
+    if (nup) {
+        bwd_zero_kernel<<<(unsigned)((nup + 255) / 256), 256, 0, st>>>(p.upper, nup);
+        int rc = check_launch("bwd_zero_kernel");
+        if (rc != HSA_OK) return rc;
+    }
+    int rc = attn_bwd_tile_launch_td<T, 64>(p, (R + TILE_Q - 1) / TILE_Q, causal != 0, st);
+    if (rc != HSA_OK) return rc;
+    const int first = level_offset(N, 4);
+    const size_t n_fin = (size_t)B * (M - first) * H * D;
+    if (n_fin) {
+        attn_bwd_tile_finish_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
+            p.upper, p.dk, p.dv, B, N, M, H, D, p.NU, first);
+        rc = check_launch("attn_bwd_tile_finish_kernel");
+    }
+    return rc;
+}
+
 }  // namespace hsa
 
 extern "C" {
@@ -635,17 +694,36 @@ int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, cons
     return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
+size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo) {
+    const bool tile = algo != HSA_ATTN_GATHER && hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
+    const size_t fl = tile ? hsa::bwd_tile_ws_floats(B, N, H, D, L) : hsa::bwd_gather_ws_floats(B, N, H, L, R);
+    return fl * sizeof(float);
+}
+
 int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk, void *dv,
-                 float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R, int causal,
-                 int dtype, void *stream) {
-    HSA_REQUIRE(q && k && v && dout && dq && dk && dv && ws_p && ws_ds, "null pointer");
+                 void *workspace, size_t workspace_bytes, int B, int N, int M, int H, int D, int L, int R,
+                 int causal, int dtype, int algo, void *stream) {
+    HSA_REQUIRE(q && k && v && dout && dq && dk && dv && workspace, "null pointer");
     HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
     HSA_REQUIRE(hsa::ilog2_exact(N) == L, "canonical table needs L == log2 N (N=%d L=%d)", N, L);
     HSA_REQUIRE(M >= 2 * N - 1, "canonical table needs M >= 2N-1 (N=%d M=%d)", N, M);
     HSA_REQUIRE(R >= 0, "bad R=%d", R);
+    HSA_REQUIRE(dtype == HSA_F32 || dtype == HSA_F16 || dtype == HSA_BF16, "unknown dtype %d", dtype);
+    HSA_REQUIRE(workspace_bytes >= hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, dtype, algo),
+                "workspace too small (%zu bytes)", workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    float *ws = (float *)workspace;
+    const bool tile_ok = hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
+    if (algo == HSA_ATTN_TILE && !tile_ok)
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "tile backward not available for N=%d D=%d L=%d R=%d dtype=%d", N, D, L, R, dtype);
+    if (tile_ok && algo != HSA_ATTN_GATHER) {
+        if (dtype == HSA_BF16)
+            return hsa::attn_bwd_tile_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);
+        return hsa::attn_bwd_tile_typed<hsa::F16>(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);
+    }
     if (2 * R + 1 + L > 64 * hsa::BWD_MAX_CHUNKS)
         return hsa::fail(HSA_ERR_UNSUPPORTED, "2R+1+L = %d slots exceeds %d", 2 * R + 1 + L, 64 * hsa::BWD_MAX_CHUNKS);
-    hipStream_t st = (hipStream_t)stream;
+    float *ws_p = ws, *ws_ds = ws + (size_t)B * N * H * (2 * R + 1 + L);
     switch (dtype) {
         case HSA_F32: return hsa::attn_bwd_typed<hsa::F32>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
         case HSA_F16: return hsa::attn_bwd_typed<hsa::F16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);

@@ -175,7 +175,7 @@ def build_parents_backward(grad_out, Q_p, K_p, V_p, K_c, V_c):
     return dq, dkp, dvp, dkc, dvc
 
 
-def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool):
+def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool, algo: str = "auto"):
     """Gradients (dQ, dK, dV) of the span attention for the canonical tables of N = Q.shape[1]."""
     _lib.require_gpu(grad_out, Q, K, V)
     grad_out, Q, K, V = (t.contiguous() for t in (grad_out, Q, K, V))
@@ -183,13 +183,14 @@ def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool):
     M = K.shape[1]
     L = N.bit_length() - 1
     R = int(window_size)
-    S = 2 * R + 1 + L
     dq, dk, dv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
-    ws = torch.empty((2, B, N, H, S), device=Q.device, dtype=torch.float32)
+    lib = _lib.lib()
+    nbytes = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(Q), _lib.algo_code(algo)))
+    ws = torch.empty((max(nbytes, 4) + 3) // 4, device=Q.device, dtype=torch.float32)
     with torch.cuda.device(Q.device):
-        rc = _lib.lib().hsa_attn_bwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(grad_out), _lib.ptr(dq),
-                                     _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws[0]), _lib.ptr(ws[1]), B, N, M, H, D,
-                                     L, R, int(bool(causal)), _lib.dtype_code(Q), _lib.stream_of(Q))
+        rc = lib.hsa_attn_bwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(grad_out), _lib.ptr(dq),
+                              _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws), ws.numel() * 4, B, N, M, H, D,
+                              L, R, int(bool(causal)), _lib.dtype_code(Q), _lib.algo_code(algo), _lib.stream_of(Q))
     _lib.check(rc, "hsa_attn_bwd")
     return dq, dk, dv
 

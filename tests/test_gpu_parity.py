@@ -372,8 +372,9 @@ def _grad_close(got, want, dtype, what):
 
 
 @pytest.mark.parametrize("case", [(2, 8, 2, 16, 2, None), (1, 64, 3, 32, 5, None), (2, 128, 4, 64, 16, None),
-                                  (1, 32, 2, 20, 0, None), (1, 16, 2, 16, 20, 40)])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+                                  (1, 32, 2, 20, 0, None), (1, 16, 2, 16, 20, 40), (1, 16, 2, 64, 3, None),
+                                  (2, 256, 3, 64, 32, 600), (1, 1024, 2, 64, 0, None), (1, 64, 12, 64, 9, None)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
     B, N, H, D, R, M = case
@@ -392,6 +393,11 @@ def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
     _grad_close(qd.grad, qr.grad, dtype, "dQ")
     _grad_close(kd.grad, kr.grad, dtype, "dK")
     _grad_close(vd.grad, vr.grad, dtype, "dV")
+    # the gather formulation explicitly (the default picks the tile kernels when eligible)
+    dq, dk, dv = fn.attention_backward(go.to(DEV), qd.detach(), kd.detach(), vd.detach(), R, causal, algo="gather")
+    _grad_close(dq, qr.grad, dtype, "dQ gather")
+    _grad_close(dk, kr.grad, dtype, "dK gather")
+    _grad_close(dv, vr.grad, dtype, "dV gather")
 
 
 def test_attention_backward_rejects_unknown_tables():
