@@ -10,8 +10,9 @@
 //      The tree key blocks are also evaluated in the other orientation (S[query, slot]), which
 //      puts the queries into the MFMA contraction: dK^T[ch, slot] = Q^T . dS, dV^T = dO^T . P.
 //      Nodes of levels 1..3 are attended only from inside the block: their rows are final and
-//      written directly.  Nodes of levels >= 4 collect from 2^(l-4) blocks: fp32 atomic adds
-//      into a small accumulation buffer (N/8 rows per sequence), converted afterwards.
+//      written directly.  A node of level l >= 4 collects from the 2^(l-4) blocks under its
+//      sibling: every block stores its fp32 partial row per level, and a small reduction kernel
+//      sums each node's contiguous run of blocks (deterministic, no atomics).
 //  (B) key-stationary, one wavefront per (batch, head, 16-leaf key block): loops over the query
 //      blocks whose window reaches the key block, rebuilds P and dS from the saved statistics
 //      and accumulates dK^T = Q^T . dS, dV^T = dO^T . P in registers.  Every leaf row of dK / dV
@@ -30,9 +31,8 @@ struct BwdTileParams {
     const uint16_t *q, *k, *v, *dout;
     uint16_t *dq, *dk, *dv;
     float *stats;   // [B, N, H, 2]: log2-domain lse, delta
-    float *upper;   // [2, B, NU, H, D] fp32 accumulators of dK, dV rows of tree levels >= 4
+    float *partial; // [2, B, N/16, H, L-4, D] fp32 per-block partial rows of dK, dV for levels >= 4
     int B, N, M, H, L, R;
-    int NU;         // rows of levels >= 4: (2N-1) - off_4 (0 when L < 5)
     int n_units;
     float scale_log2e, scale;
 };
@@ -359,23 +359,17 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
                 }
             }
         }
-        // slots of levels >= 4 accumulate over blocks: fp32 atomics
+        // slots of levels >= 4 collect from several blocks: this block's partial rows
         const int lvl = t == 0 ? (r16 >= 14 ? 4 + (r16 - 14) : -1) : 6 + r16;
         if (lvl >= 4 && lvl < L) {
-            const int row = level_offset(N, lvl) + ((q0 >> lvl) ^ 1);
-            const size_t uo = (((size_t)b * p.NU + (row - level_offset(N, 4))) * H + h) * D;
-            float *uk = p.upper + uo;
-            float *uv = p.upper + (size_t)p.B * p.NU * H * D + uo;
-            const bool live = !CAUSAL || ((q0 >> lvl) & 1);
-            if (live) {
+            const size_t po = ((((size_t)b * NB + blk) * H + h) * (L - 4) + (lvl - 4)) * D;
+            float *pk = p.partial + po;
+            float *pv = p.partial + (size_t)p.B * NB * H * (L - 4) * D + po;
 #pragma unroll
-                for (int j = 0; j < NJ; ++j)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1) + i;
-                        unsafeAtomicAdd(uk + ch, tk[j][i]);
-                        unsafeAtomicAdd(uv + ch, tv[j][i]);
-                    }
+            for (int j = 0; j < NJ; ++j) {
+                const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                *reinterpret_cast<f32x4 *>(pk + ch) = tk[j];
+                *reinterpret_cast<f32x4 *>(pv + ch) = tv[j];
             }
         }
     }
@@ -493,25 +487,40 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
     }
 }
 
-// rows of tree levels >= 4: fp32 accumulators -> element type; the root and any extra rows get zeros
+// Rows of tree levels >= 4 (and anything above row 2N-2): node (l, p) sums the partial rows of the
+// 2^(l-4) query blocks under its sibling; nodes nobody attends (the root, right-hand nodes when
+// causal, rows past 2N-1) get zeros.  One thread per (batch, row, head, channel).
 template <typename T>
-__global__ void attn_bwd_tile_finish_kernel(const float *__restrict__ upper, uint16_t *__restrict__ dk,
-                                            uint16_t *__restrict__ dv, int B, int N, int M, int H, int D, int NU,
-                                            int first_upper_row) {
-    const size_t per_b = (size_t)(M - first_upper_row) * H * D;
+__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ dk,
+                                            uint16_t *__restrict__ dv, int B, int N, int M, int H, int D, int L,
+                                            int causal, int first_row) {
+    const size_t per_b = (size_t)(M - first_row) * H * D;
     const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (size_t)B * per_b) return;
     const int b = (int)(t / per_b);
     const size_t r = t % per_b;
-    const int row = first_upper_row + (int)(r / ((size_t)H * D));
-    const size_t hd = r % ((size_t)H * D);
+    const int row = first_row + (int)(r / ((size_t)H * D));
+    const int h = (int)((r / D) % H);
+    const int d = (int)(r % D);
     float vk = 0.f, vv = 0.f;
-    if (row < 2 * N - 2) {  // below the root
-        const size_t uo = ((size_t)b * NU + (row - first_upper_row)) * H * D + hd;
-        vk = upper[uo];
-        vv = upper[(size_t)B * NU * H * D + uo];
+    if (row < 2 * N - 2) {
+        int lvl = 4;
+        while (row >= level_offset(N, lvl + 1)) ++lvl;
+        const int pidx = row - level_offset(N, lvl);
+        if (!causal || (pidx & 1) == 0) {
+            const int NB = N / TILE_Q;
+            const int nblk = 1 << (lvl - 4);
+            const int blk0 = (pidx ^ 1) << (lvl - 4);
+            const size_t stride = (size_t)H * (L - 4) * D;
+            const float *pk = partial + (((size_t)b * NB + blk0) * H + h) * (L - 4) * D + (size_t)(lvl - 4) * D + d;
+            const float *pv = pk + (size_t)B * NB * H * (L - 4) * D;
+            for (int i = 0; i < nblk; ++i) {
+                vk += pk[(size_t)i * stride];
+                vv += pv[(size_t)i * stride];
+            }
+        }
     }
-    const size_t o = ((size_t)b * M + row) * H * D + hd;
+    const size_t o = ((size_t)b * M + row) * H * D + (size_t)h * D + d;
     dk[o] = from_float<T>(vk);
     dv[o] = from_float<T>(vv);
 }

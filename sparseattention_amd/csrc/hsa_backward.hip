@@ -621,11 +621,6 @@ __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, ty
 }
 
 // ---------------------------------------------------------------- tile backward dispatch
-__global__ void bwd_zero_kernel(float *p, size_t n) {
-    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t < n) p[t] = 0.f;
-}
-
 static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype) {
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 64) return false;
@@ -637,9 +632,9 @@ static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype)
 static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
     return 2 * (size_t)B * N * H * (2 * R + 1 + L);
 }
-static int bwd_tile_nu(int N, int L) { return L >= 4 ? (2 * N - 1) - level_offset(N, 4) : 0; }
 static size_t bwd_tile_ws_floats(int B, int N, int H, int D, int L) {
-    return (size_t)B * N * H * 2 + 2 * (size_t)B * bwd_tile_nu(N, L) * H * D;
+    const size_t lv = L > 4 ? L - 4 : 0;
+    return (size_t)B * N * H * 2 + 2 * (size_t)B * (N / TILE_Q) * H * lv * D;
 }
 
 template <typename T>
@@ -650,28 +645,21 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v; p.dout = (const uint16_t *)dout;
     p.dq = (uint16_t *)dq; p.dk = (uint16_t *)dk; p.dv = (uint16_t *)dv;
     p.stats = ws;
-    p.upper = ws + (size_t)B * N * H * 2;
+    p.partial = ws + (size_t)B * N * H * 2;
     p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
-    p.NU = bwd_tile_nu(N, L);
     const long units = (long)B * (N / TILE_Q) * H;
     if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.n_units = (int)units;
     p.scale = 1.0f / sqrtf((float)D);
     p.scale_log2e = 1.4426950408889634f * p.scale;
-    const size_t nup = 2 * (size_t)B * p.NU * H * D;
-    if (nup) {
-        bwd_zero_kernel<<<(unsigned)((nup + 255) / 256), 256, 0, st>>>(p.upper, nup);
-        int rc = check_launch("bwd_zero_kernel");
-        if (rc != HSA_OK) return rc;
-    }
     int rc = attn_bwd_tile_launch_td<T, 64>(p, (R + TILE_Q - 1) / TILE_Q, causal != 0, st);
     if (rc != HSA_OK) return rc;
     const int first = level_offset(N, 4);
     const size_t n_fin = (size_t)B * (M - first) * H * D;
     if (n_fin) {
-        attn_bwd_tile_finish_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
-            p.upper, p.dk, p.dv, B, N, M, H, D, p.NU, first);
-        rc = check_launch("attn_bwd_tile_finish_kernel");
+        attn_bwd_tile_reduce_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
+            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first);
+        rc = check_launch("attn_bwd_tile_reduce_kernel");
     }
     return rc;
 }
