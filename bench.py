@@ -221,6 +221,17 @@ def main():
     attn_avg_ms = launches_ms(lib.hsa_attn_fwd, aargs)
     tree_b2b_ms = launches_ms(lib.hsa_build_tree_fwd, targs)
 
+    # --- backward of the span attention (next-row kernel), same rotation of inputs ----------------
+    gq = torch.randn(B, N, H, D, device=dev).to(torch.bfloat16)
+    dq_, dk_, dv_ = torch.empty_like(gq), torch.empty_like(sets[0]["kfull"]), torch.empty_like(sets[0]["kfull"])
+    wsb = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.HSA_BF16, _lib.ATTN_AUTO))
+    wsp = torch.empty(max(wsb, 4) // 4 + 1, device=dev, dtype=torch.float32)
+    bargs = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(gq), P(dq_), P(dk_), P(dv_), P(wsp), wsp.numel() * 4,
+              B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st) for s in sets]
+    for i in range(3):
+        assert lib.hsa_attn_bwd(*bargs[i % nsets]) == 0, lib.hsa_last_error()
+    attn_bwd_ms = launches_ms(lib.hsa_attn_bwd, bargs)
+
     # --- the same K steps with an event pair around every attention launch (each pair adds
     #     ~5 us of idle time around the kernel, so this is reported as detail only) ----------
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(K)]
@@ -275,6 +286,8 @@ def main():
                    "tree_build_avg_launch_ms": tree_b2b_ms,
                    "tree_algorithmic_bytes": tree_bytes,
                    "tree_GBps": tree_bytes / (tree_b2b_ms * 1e-3) / 1e9,
+                   "attn_backward_avg_ms": attn_bwd_ms,
+                   "attn_backward_algorithmic_bytes": e * B * H * D * (2 * N + 2 * M + N + 2 * M),
                    "attn_ms_in_step_event_pair_avg": attn_instep_avg_ms,
                    "attn_ms_in_step_event_pair_median": attn_instep_med_ms},
     }

@@ -208,31 +208,34 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
         for (int i = 0; i < NLD; ++i)
             dst[i] = *reinterpret_cast<const u32x4_t *>(base + (size_t)(rows[i] < 0 ? q0 : rows[i]) * rs);
     };
-    u32x4_t rQ[NLD], rG[NLD], rK[NKB][NLD], rV[NKB][NLD];
-    load_block(Qb, q0, rQ);
-    load_block(Gb, q0, rG);
-#pragma unroll
-    for (int c = 0; c < NKL; ++c) {
-        int kb = blk - NBW + c;
-        kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
-        load_block(Kb, kb * TILE_Q, rK[c]);
-        load_block(Vb, kb * TILE_Q, rV[c]);
-    }
-    load_rows(Kb, t_row, rK[NKL]);
-    load_rows(Vb, t_row, rV[NKL]);
-    load_rows(Kb, u_row, rK[NKL + 1]);
-    load_rows(Vb, u_row, rV[NKL + 1]);
-
-    // ---- operand forms ------------------------------------------------------------------------
+    // ---- loads and operand forms (each block: rows -> LDS -> MFMA pieces) -----------------------
     u32x4_t Qf[KS], Gf[KS], Kc[NKB][KS], Vc[NKB][KS];
-    bt.put(0, rQ);
-    bt.put(1, rG);
-    bt.get(0, Qf);
-    bt.get(1, Gf);
+    {
+        u32x4_t rQ[NLD], rG[NLD];
+        load_block(Qb, q0, rQ);
+        load_block(Gb, q0, rG);
+        bt.put(0, rQ);
+        bt.put(1, rG);
+        bt.get(0, Qf);
+        bt.get(1, Gf);
+    }
 #pragma unroll
     for (int c = 0; c < NKB; ++c) {
-        bt.put(2, rK[c]);
-        bt.put(3, rV[c]);
+        u32x4_t rK[NLD], rV[NLD];
+        if (c < NKL) {
+            int kb = blk - NBW + c;
+            kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
+            load_block(Kb, kb * TILE_Q, rK);
+            load_block(Vb, kb * TILE_Q, rV);
+        } else if (c == NKL) {
+            load_rows(Kb, t_row, rK);
+            load_rows(Vb, t_row, rV);
+        } else {
+            load_rows(Kb, u_row, rK);
+            load_rows(Vb, u_row, rV);
+        }
+        bt.put(2, rK);
+        bt.put(3, rV);
         bt.get(2, Kc[c]);
         bt.get(3, Vc[c]);
     }

@@ -1,4 +1,4 @@
-// Instantiates the tile backward kernels of one element type (head_dim 64).
+// Instantiates the tile backward kernels of one (element type, head_dim) pair.
 #pragma once
 #include "hsa_attn_bwd_tile.h"
 
