@@ -102,7 +102,7 @@ def lm_forward_bench(args):
         ms = (time.perf_counter() - t0) * 1e3 / K
         # time share of the two custom ops: the same forward with an event pair around each call
         spans = {"build_parent_nodes": [], "hierarchical_attention": []}
-        orig_b, orig_h = attn_mod.build_parent_nodes, attn_mod.hierarchical_attention
+        orig_b, orig_h = attn_mod.build_parents_forward, attn_mod.hierarchical_attention
 
         def timed(name, f):
             def g(*a, **k):
@@ -114,11 +114,11 @@ def lm_forward_bench(args):
                 return r
             return g
 
-        attn_mod.build_parent_nodes = timed("build_parent_nodes", orig_b)
+        attn_mod.build_parents_forward = timed("build_parent_nodes", orig_b)
         attn_mod.hierarchical_attention = timed("hierarchical_attention", orig_h)
         model(tok)
         torch.cuda.synchronize()
-        attn_mod.build_parent_nodes, attn_mod.hierarchical_attention = orig_b, orig_h
+        attn_mod.build_parents_forward, attn_mod.hierarchical_attention = orig_b, orig_h
     share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",

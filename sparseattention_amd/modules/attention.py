@@ -13,7 +13,7 @@ from typing import List, Optional
 import torch
 import torch.nn as nn
 
-from ..ops.functional import build_parent_nodes, hierarchical_attention
+from ..ops.functional import build_parent_nodes, build_parents_forward, hierarchical_attention
 from ..ops.topology import build_tree_topology
 
 
@@ -81,16 +81,27 @@ class HierarchicalAttention(nn.Module):
         k_lv = torch.split(self._heads(self.Wk_y(y_in)), self.sizes, dim=1)
         v_lv = torch.split(self._heads(self.Wv_y(y_in)), self.sizes, dim=1)
 
-        levels, src = [], x
+        # Without autograd the level outputs go straight into one [B, N-1, D] buffer (no
+        # concatenation afterwards); with autograd each level is a differentiable op.
+        direct = not (torch.is_grad_enabled() and (x.requires_grad or y_in.requires_grad
+                                                    or self.Wq_y.weight.requires_grad))
+        y_new = torch.empty((B, N - 1, D), dtype=x.dtype, device=x.device) if direct else None
+        levels, src, off = [], x, 0
         for lvl, P in enumerate(self.sizes):
             k_c = self._heads(self.Wk_y(src))
             v_c = self.dropout(self._heads(self.Wv_y(src)))
             if lvl == 0:
                 v_c = self.dropout(v_c)  # the leaf values pass through dropout twice
-            merged = build_parent_nodes(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c).reshape(B, P, D)
-            levels.append(merged)
-            src = merged
-        return self.out_proj_y(torch.cat(levels, dim=1))
+            if direct:
+                dst = y_new[:, off:off + P]
+                build_parents_forward(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c,
+                                      out=dst.view(B, P, self.num_heads, self.head_dim))
+                src = dst
+            else:
+                src = build_parent_nodes(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c).reshape(B, P, D)
+                levels.append(src)
+            off += P
+        return self.out_proj_y(y_new if direct else torch.cat(levels, dim=1))
 
     # -- top-down: span nodes -> leaves -------------------------------------------
     def update_X_from_Y(self, x: torch.Tensor, y: torch.Tensor,

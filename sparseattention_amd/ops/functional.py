@@ -96,32 +96,49 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
     return (out, weights) if return_weights else out
 
 
-def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False):
-    """One level of the parent build on [B,P,H,D] / [B,2P,H,D] tensors."""
-    _lib.require_gpu(Q_p, K_p, V_p, K_c, V_c)
-    Q_p, K_p, V_p, K_c, V_c = (t.contiguous() for t in (Q_p, K_p, V_p, K_c, V_c))
+def _rows_dense(t: torch.Tensor) -> bool:
+    B, rows, H, D = t.shape
+    return t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D
+
+
+def _batch_stride(t: torch.Tensor) -> int:
+    """Element stride between batches of a [B, rows, H, D] tensor whose rows are dense."""
+    B, rows, H, D = t.shape
+    assert _rows_dense(t), "rows of the tensor must be dense [rows, H, D]"
+    return t.stride(0) if B > 1 else rows * H * D
+
+
+def _dense_rows(t: torch.Tensor) -> torch.Tensor:
+    """The tensor itself when each batch's rows are dense (a level slice of a larger buffer
+    qualifies: only the batch stride differs), else a contiguous copy."""
+    return t if _rows_dense(t) else t.contiguous()
+
+
+def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False,
+                          out: Optional[torch.Tensor] = None):
+    """One level of the parent build on [B,P,H,D] / [B,2P,H,D] tensors.  Inputs may be level
+    slices of larger buffers (dense rows, any batch stride); `out` may be such a slice too."""
+    _lib.require_gpu(Q_p, K_p, V_p, K_c, V_c, out)
+    Q_p, K_p, V_p, K_c, V_c = (_dense_rows(t) for t in (Q_p, K_p, V_p, K_c, V_c))
     B, P, H, D = Q_p.shape
     assert K_c.shape[1] == 2 * P, "Child count mismatch"
     assert K_p.shape == Q_p.shape and V_p.shape == Q_p.shape, "parent K/V shape mismatch"
     assert V_c.shape == K_c.shape and K_c.shape[0] == B and K_c.shape[2:] == Q_p.shape[2:], \
         "child K/V shape mismatch"
     assert Q_p.dtype == K_p.dtype == V_p.dtype == K_c.dtype == V_c.dtype, "dtype mismatch"
-    out = torch.empty_like(Q_p)
+    if out is None:
+        out = torch.empty((B, P, H, D), dtype=Q_p.dtype, device=Q_p.device)
+    else:
+        assert out.shape == (B, P, H, D) and out.dtype == Q_p.dtype and _rows_dense(out)
     weights = torch.empty((B, P, H, 3), device=Q_p.device, dtype=Q_p.dtype) if return_weights else None
     with torch.cuda.device(Q_p.device):
         rc = _lib.lib().hsa_build_parents_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
-            _lib.ptr(weights), B, P, H, D, 0, 0, 0, 0, 0, 0, _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
+            _lib.ptr(weights), B, P, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
+            _batch_stride(K_c), _batch_stride(V_c), _batch_stride(out), _lib.dtype_code(Q_p),
+            _lib.stream_of(Q_p))
     _lib.check(rc, "hsa_build_parents_fwd")
     return (out, weights) if return_weights else out
-
-
-def _batch_stride(t: torch.Tensor) -> int:
-    """Element stride between batches of a [B, rows, H, D] tensor whose rows are dense."""
-    B, rows, H, D = t.shape
-    assert t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D, \
-        "rows of the tensor must be dense [rows, H, D]"
-    return t.stride(0) if B > 1 else rows * H * D
 
 
 def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None,
