@@ -517,7 +517,16 @@ __global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, u
             const size_t stride = (size_t)H * (L - 4) * D;
             const float *pk = partial + (((size_t)b * NB + blk0) * H + h) * (L - 4) * D + (size_t)(lvl - 4) * D + d;
             const float *pv = pk + (size_t)B * NB * H * (L - 4) * D;
-            for (int i = 0; i < nblk; ++i) {
+            // eight independent loads in flight per round trip (the top nodes sum up to N/32 rows)
+            int i = 0;
+            for (; i + 8 <= nblk; i += 8) {
+                float a[8], c[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { a[u] = pk[(size_t)(i + u) * stride]; c[u] = pv[(size_t)(i + u) * stride]; }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) { vk += a[u]; vv += c[u]; }
+            }
+            for (; i < nblk; ++i) {
                 vk += pk[(size_t)i * stride];
                 vv += pv[(size_t)i * stride];
             }
