@@ -322,10 +322,12 @@ def test_transformer_lm_vs_oracle(activation):
 
 
 # ---------------------------------------------------------------- long-sequence stress (size-independent checks)
-def test_cfg5_long_sequence_properties():
-    """B1 H16 N65536 D128 bf16 R32: too large for the gather oracle in seconds, so check what
+@pytest.mark.parametrize("shape", [(1, 16, 65536, 128, 32), (1, 1, 1 << 20, 64, 16)])
+def test_long_sequence_properties(shape):
+    """B1 H16 N65536 D128 bf16 R32 (the long-sequence stress shape) and a 2^20-leaf tree (20 levels,
+    the far tree block nearly full): too large for the gather oracle in seconds, so check what
     the mathematics fixes plus a brute-force sample of rows."""
-    B, H, N, D, R = 1, 16, 65536, 128, 32
+    B, H, N, D, R = shape
     g = torch.Generator().manual_seed(0)
     q = torch.randn(B, N, H, D, generator=g).to(torch.bfloat16)
     k = torch.randn(B, 2 * N - 1, H, D, generator=g).to(torch.bfloat16)
@@ -340,8 +342,8 @@ def test_cfg5_long_sequence_properties():
     oc = sa.hierarchical_attention(qd, kd, const, t["forward_idx"], t["backward_gather"], t["forward_mask"], R)
     assert (oc.float() - 0.5).abs().max() < 4e-3
     # brute force on a sample of rows spread over the sequence (first, last, block borders)
-    rows = sorted(set([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 1023, 1024, 4095, 4096, 32767, 32768, 65534, 65535]
-                      + list(range(7, N, 4099))))
+    rows = sorted(set([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 1023, 1024, 4095, 4096, 32767, 32768, 65534, 65535,
+                       N // 2 - 1, N // 2, N - 2, N - 1] + list(range(7, N, N // 16 + 3))))
     o = oracle.topology_tables(N, True)
     sel = torch.tensor(rows)
     outs = []
