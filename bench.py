@@ -135,8 +135,9 @@ def lm_forward_bench(args):
 def main():
     args = parse()
     if args.gpus != 1:
-        print("bench.py measures one GPU only: this build has no multi-GPU path (every (batch, head) "
-              "is independent; see DESIGN.md for how it would shard). Re-run with --gpus 1.", file=sys.stderr)
+        print("bench.py measures one GPU only: this build has no multi-GPU path (every (batch, head) is "
+              "independent, so the path would shard over batch or heads without any exchange). "
+              "Re-run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
     import torch
     from sparseattention_amd import _lib
