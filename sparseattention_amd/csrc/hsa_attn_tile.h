@@ -34,6 +34,8 @@
 
 #include "hsa_common.h"
 
+#include <type_traits>
+
 namespace hsa {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -99,6 +101,7 @@ struct TileParams {
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
     int xcd_swizzle;
+    int alternate;    // neighbouring strips walk in opposite directions
     float scale_log2e;
 };
 
@@ -123,7 +126,6 @@ attn_tile_kernel(TileParams p) {
     constexpr int KS = D / 32;                         // 32-channel steps of the QK contraction
     constexpr int NJ = D / 16;                         // 16-channel output tiles
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // leaf key blocks per query block
-    constexpr int NEWC = NKL - 1;                      // the leaf block that enters each step
     constexpr int CPR = D / 8;                         // 16-byte pieces per head-row
     constexpr int RPI = 64 / CPR;                      // rows covered by one load instruction
     constexpr int NLD = TILE_Q / RPI;                  // load instructions per 16-row block (= 2*KS)
@@ -296,10 +298,20 @@ attn_tile_kernel(TileParams p) {
     struct Stage {
         u32x4_t q[NLD], k[NLD], v[NLD], kt[NLD], vt[NLD];
     };
+    // One strip, walked upwards (REV = false) or downwards (REV = true).  Neighbouring strips
+    // walk in opposite directions, so the leaf block that two strips share (the last block of
+    // one, the left neighbour of the other's first) is fetched by both at the same moment and
+    // the second fetch hits in L2 instead of going back to memory.
+    // Kl[c] / Vl[c] hold leaf block (blk - NBW + c) of the query block being processed; the
+    // block that enters per step is the top one walking upwards, the bottom one downwards.
+    auto run = [&](auto rev_tag) {
+    constexpr bool REV = decltype(rev_tag)::value;
+    constexpr int NEWI = REV ? 0 : NKL - 1;
+    auto seq = [&](int it) { return REV ? blk0 + SB - 1 - it : blk0 + it; };
     auto request = [&](Stage &sg, int blk) {
         const int q0 = blk * TILE_Q;
         load_block(Qb, q0, sg.q);
-        const int row0 = leaf_row0(blk + (CAUSAL ? 0 : NBW));
+        const int row0 = leaf_row0(blk - NBW + NEWI);
         load_block(Kb, row0, sg.k);
         load_block(Vb, row0, sg.v);
         load_near(Kb, q0, sg.kt);
@@ -310,9 +322,9 @@ attn_tile_kernel(TileParams p) {
     constexpr int AHEAD = (D <= 64) ? 2 : 1;
     Stage st[SB];
 #pragma unroll
-    for (int i = 0; i < AHEAD && i < SB; ++i) request(st[i], blk0 + i);
+    for (int i = 0; i < AHEAD && i < SB; ++i) request(st[i], seq(i));
 
-    // ---- per-strip operands: far tree block, leaf blocks left of the first query block ----
+    // ---- per-strip operands: far tree block, leaf blocks carried into the first query block ----
     u32x4_t Ku[KS];
     u32x2_t Vu[NJ];
     {
@@ -328,8 +340,9 @@ attn_tile_kernel(TileParams p) {
     u32x4_t Kl[NKL][KS];
     u32x2_t Vl[NKL][NJ];
 #pragma unroll
-    for (int c = 0; c < NKL - 1; ++c) {
-        const int row0 = leaf_row0(blk0 - NBW + c);
+    for (int c = 0; c < NKL; ++c) {
+        if (c == NEWI) continue;
+        const int row0 = leaf_row0(seq(0) - NBW + c);
         u32x4_t rk[NLD], rv[NLD], vop[KS];
         load_block(Kb, row0, rk);
         load_block(Vb, row0, rv);
@@ -352,7 +365,7 @@ attn_tile_kernel(TileParams p) {
         // this block's raw registers are consumed: request a later block's
         if (next_blk >= 0) request(nsg, next_blk);
         lds_get(0, Qf);
-        lds_get(1, Kl[NEWC]);
+        lds_get(1, Kl[NEWI]);
         lds_get(2, Vn);
         lds_get(3, Kt);
         lds_get(4, Vtn);
@@ -374,7 +387,7 @@ attn_tile_kernel(TileParams p) {
         }
         // new value blocks into "lane = channel, regs = keys" form
         u32x2_t Vt[NJ];
-        transpose_v(Vn, Vl[NEWC]);
+        transpose_v(Vn, Vl[NEWI]);
         transpose_v(Vtn, Vt);
 
         float sc[NKL + 2][4];
@@ -453,20 +466,34 @@ attn_tile_kernel(TileParams p) {
         }
 
         // slide the leaf window by one block
+        if (REV) {
 #pragma unroll
-        for (int c = 0; c + 1 < NKL; ++c) {
+            for (int c = NKL - 1; c > 0; --c) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) Kl[c][ks] = Kl[c + 1][ks];
+                for (int ks = 0; ks < KS; ++ks) Kl[c][ks] = Kl[c - 1][ks];
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) Vl[c][j] = Vl[c + 1][j];
+                for (int j = 0; j < NJ; ++j) Vl[c][j] = Vl[c - 1][j];
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c + 1 < NKL; ++c) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) Kl[c][ks] = Kl[c + 1][ks];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) Vl[c][j] = Vl[c + 1][j];
+            }
         }
     };
 
 #pragma unroll
     for (int it = 0; it < SB; ++it) {
-        if (it + AHEAD < SB) process(st[it], blk0 + it, st[it + AHEAD], blk0 + it + AHEAD);
-        else process(st[it], blk0 + it, st[it], -1);
+        if (it + AHEAD < SB) process(st[it], seq(it), st[it + AHEAD], seq(it + AHEAD));
+        else process(st[it], seq(it), st[it], -1);
     }
+    };  // run
+
+    if (p.alternate && (s & 1)) run(std::true_type{});
+    else run(std::false_type{});
 }
 
 template <typename T, int D>

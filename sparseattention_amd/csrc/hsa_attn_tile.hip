@@ -42,6 +42,8 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     p.n_units = (int)units;
     p.xcd_swizzle = 1;
     if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) p.xcd_swizzle = atoi(e);
+    p.alternate = 1;
+    if (const char *e = getenv("HSA_ATTN_TILE_ALT")) p.alternate = atoi(e);
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
     int wpb = 8;
     if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
