@@ -100,9 +100,11 @@ def lm_forward_bench(args):
             model(tok)
         torch.cuda.synchronize()
         ms = (time.perf_counter() - t0) * 1e3 / K
-        # time share of the two custom ops: the same forward with an event pair around each call
-        spans = {"build_parent_nodes": [], "hierarchical_attention": []}
-        orig_b, orig_h = attn_mod.build_parents_forward, attn_mod.hierarchical_attention
+        # time share of the tree side (cross_update_Y: projections + one kernel per level) and of
+        # the span attention op: the same forward with an event pair around each call
+        spans = {"cross_update_Y": [], "hierarchical_attention": []}
+        cls = attn_mod.HierarchicalAttention
+        orig_c, orig_h = cls.cross_update_Y, attn_mod.hierarchical_attention
 
         def timed(name, f):
             def g(*a, **k):
@@ -114,11 +116,11 @@ def lm_forward_bench(args):
                 return r
             return g
 
-        attn_mod.build_parents_forward = timed("build_parent_nodes", orig_b)
+        cls.cross_update_Y = timed("cross_update_Y", orig_c)
         attn_mod.hierarchical_attention = timed("hierarchical_attention", orig_h)
         model(tok)
         torch.cuda.synchronize()
-        attn_mod.build_parents_forward, attn_mod.hierarchical_attention = orig_b, orig_h
+        cls.cross_update_Y, attn_mod.hierarchical_attention = orig_c, orig_h
     share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
@@ -126,9 +128,9 @@ def lm_forward_bench(args):
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "cfg4: decoder LM forward, random init, eval mode"},
-        "detail": {"ms_in_build_parent_nodes_event_pairs": share["build_parent_nodes"],
+        "detail": {"ms_in_cross_update_Y_event_pairs": share["cross_update_Y"],
                    "ms_in_hierarchical_attention_event_pairs": share["hierarchical_attention"],
-                   "calls_build_parent_nodes": len(spans["build_parent_nodes"]),
+                   "calls_cross_update_Y": len(spans["cross_update_Y"]),
                    "calls_hierarchical_attention": len(spans["hierarchical_attention"])}}))
 
 

@@ -93,6 +93,25 @@ int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const 
                           int64_t vc_bs, int64_t out_bs, int dtype, void *stream);
 
 /*
+ * One level of the parent build whose operands are column slices of wider matrices: the level
+ * step of HierarchicalAttention.cross_update_Y
+ * (hierarchical_attention/modules/attention.py:119-157) once the projections that feed it are
+ * fused, so that q/k/v of the parents are thirds of one [B, N-1, 3*H*D] projection and the
+ * children's k/v are halves of one [B, 2P, 2*H*D] projection.  Same arithmetic as
+ * hsa_build_parents_fwd.
+ *
+ *   batch_strides, row_strides   host arrays of 7 element counts in the order
+ *                                qp, kp, vp, kc, vc, out, out2; an entry of 0, or a NULL
+ *                                array, means dense (rows H*D apart, batches rows*row apart)
+ *   out2                         optional second copy of the result (NULL to skip), e.g. the
+ *                                level's slice of the concatenated [B, N-1, H*D] result
+ */
+int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp, const void *kc,
+                                  const void *vc, void *out, void *out2, int B, int P, int H,
+                                  int D, const int64_t *batch_strides, const int64_t *row_strides,
+                                  int dtype, void *stream);
+
+/*
  * Whole tree in one call: level 1 from the leaves, every further level from the
  * previous level's output used as both child K and child V (the composition
  * Out_l = build_parent_nodes(Qp_l, Kp_l, Vp_l, Out_{l-1}, Out_{l-1}) of the op at

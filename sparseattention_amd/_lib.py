@@ -36,6 +36,8 @@ def _declare(lib):
     lib.hsa_attn_fwd_uses_tile.restype = I
     lib.hsa_build_parents_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 6 + [I, P]
     lib.hsa_build_parents_fwd.restype = I
+    lib.hsa_build_parents_strided_fwd.argtypes = [P] * 7 + [I] * 4 + [P, P, I, P]
+    lib.hsa_build_parents_strided_fwd.restype = I
     lib.hsa_build_tree_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 7 + [I, P]
     lib.hsa_build_tree_fwd.restype = I
     lib.hsa_topology_host.argtypes = [I, I, P, P, P]

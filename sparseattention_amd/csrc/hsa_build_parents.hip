@@ -63,6 +63,14 @@ __device__ __forceinline__ void softmax3(float s0, float s1, float s2, float &w0
     }
 }
 
+// Batch and row strides (in elements) of the seven operands of one level, in the order
+// qp, kp, vp, kc, vc, out, out2.  A row stride wider than H*D reads a column slice of a
+// wider matrix, e.g. one third of a fused q/k/v projection.
+struct LevelStrides {
+    int64_t bs[7];
+    int64_t rs[7];
+};
+
 // CH = number of VEC-chunks each lane holds (D <= G * VEC * CH).
 template <typename T, int VEC, int CH>
 __global__ void __launch_bounds__(256)
@@ -70,8 +78,7 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
                      const typename T::storage *__restrict__ Vp, const typename T::storage *__restrict__ Kc,
                      const typename T::storage *__restrict__ Vc, typename T::storage *__restrict__ Out,
                      typename T::storage *__restrict__ Out2, typename T::storage *__restrict__ Wt, int B,
-                     int P, int H, int D, int G, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
-                     int64_t vc_bs, int64_t out_bs, int64_t out2_bs, float scale) {
+                     int P, int H, int D, int G, LevelStrides sd, float scale) {
     const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long unit = tid / G;
     const int gl = (int)(tid % G);
@@ -81,16 +88,14 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
     const int h = (int)(u % H);
     const int i = (int)((u / H) % P);
     const int b = (int)(u / ((long)H * P));
-    const size_t prow = ((size_t)i * H + h) * D;
-    const size_t c0row = ((size_t)(2 * i) * H + h) * D;
-    const size_t c1row = c0row + (size_t)H * D;
-    const typename T::storage *q = Qp + (size_t)b * qp_bs + prow;
-    const typename T::storage *kp = Kp + (size_t)b * kp_bs + prow;
-    const typename T::storage *vp = Vp + (size_t)b * vp_bs + prow;
-    const typename T::storage *k0 = Kc + (size_t)b * kc_bs + c0row;
-    const typename T::storage *k1 = Kc + (size_t)b * kc_bs + c1row;
-    const typename T::storage *v0 = Vc + (size_t)b * vc_bs + c0row;
-    const typename T::storage *v1 = Vc + (size_t)b * vc_bs + c1row;
+    const size_t hd = (size_t)h * D;
+    const typename T::storage *q = Qp + (size_t)b * sd.bs[0] + (size_t)i * sd.rs[0] + hd;
+    const typename T::storage *kp = Kp + (size_t)b * sd.bs[1] + (size_t)i * sd.rs[1] + hd;
+    const typename T::storage *vp = Vp + (size_t)b * sd.bs[2] + (size_t)i * sd.rs[2] + hd;
+    const typename T::storage *k0 = Kc + (size_t)b * sd.bs[3] + (size_t)(2 * i) * sd.rs[3] + hd;
+    const typename T::storage *k1 = k0 + sd.rs[3];
+    const typename T::storage *v0 = Vc + (size_t)b * sd.bs[4] + (size_t)(2 * i) * sd.rs[4] + hd;
+    const typename T::storage *v1 = v0 + sd.rs[4];
 
     float fvp[CH][VEC], fv0[CH][VEC], fv1[CH][VEC];
     float s0 = 0.f, s1 = 0.f, s2 = 0.f;
@@ -120,8 +125,8 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
     float w0, w1, w2;
     softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
     if (!active) return;
-    typename T::storage *o = Out + (size_t)b * out_bs + prow;
-    typename T::storage *o2 = Out2 ? Out2 + (size_t)b * out2_bs + prow : nullptr;
+    typename T::storage *o = Out + (size_t)b * sd.bs[5] + (size_t)i * sd.rs[5] + hd;
+    typename T::storage *o2 = Out2 ? Out2 + (size_t)b * sd.bs[6] + (size_t)i * sd.rs[6] + hd : nullptr;
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int d = (c * G + gl) * VEC;
@@ -144,8 +149,7 @@ build_parents_kernel(const typename T::storage *__restrict__ Qp, const typename 
 template <typename T, int VEC>
 static int build_parents_launch(const void *qp, const void *kp, const void *vp, const void *kc,
                                 const void *vc, void *out, void *out2, void *weights, int B, int P, int H, int D,
-                                int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs,
-                                int64_t out_bs, int64_t out2_bs, hipStream_t st) {
+                                const LevelStrides &sd, hipStream_t st) {
     using S = typename T::storage;
     const int chunks = (D + VEC - 1) / VEC;  // D % VEC == 0 guaranteed by the caller when VEC > 1
     int G = 1;
@@ -159,7 +163,7 @@ static int build_parents_launch(const void *qp, const void *kp, const void *vp, 
 #define HSA_BPN_LAUNCH(CHN)                                                                        \
     build_parents_kernel<T, VEC, CHN><<<(unsigned)blocks, block, 0, st>>>(                         \
         (const S *)qp, (const S *)kp, (const S *)vp, (const S *)kc, (const S *)vc, (S *)out,       \
-        (S *)out2, (S *)weights, B, P, H, D, G, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, scale)
+        (S *)out2, (S *)weights, B, P, H, D, G, sd, scale)
     if (CH == 1) HSA_BPN_LAUNCH(1);
     else if (CH == 2) HSA_BPN_LAUNCH(2);
     else if (CH <= 4) HSA_BPN_LAUNCH(4);
@@ -508,37 +512,42 @@ int build_tree_dispatch(const void *qp, const void *kp, const void *vp, const vo
 template <typename T>
 static int build_parents_typed(const void *qp, const void *kp, const void *vp, const void *kc,
                                const void *vc, void *out, void *out2, void *weights, int B, int P, int H,
-                               int D, int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kc_bs,
-                               int64_t vc_bs, int64_t out_bs, int64_t out2_bs, hipStream_t st) {
+                               int D, const LevelStrides &sd, hipStream_t st) {
     constexpr int VEC = 16 / (int)sizeof(typename T::storage);
     const uintptr_t align = (uintptr_t)qp | (uintptr_t)kp | (uintptr_t)vp | (uintptr_t)kc | (uintptr_t)vc |
                             (uintptr_t)out | (uintptr_t)out2;
-    const int64_t strides = qp_bs | kp_bs | vp_bs | kc_bs | vc_bs | out_bs | out2_bs;
+    int64_t strides = 0;
+    for (int i = 0; i < 7; ++i) strides |= sd.bs[i] | sd.rs[i];
     if (D % VEC == 0 && (align & 15) == 0 && (strides % VEC) == 0)
-        return build_parents_launch<T, VEC>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs,
-                                            vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
-    return build_parents_launch<T, 1>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs,
-                                      kc_bs, vc_bs, out_bs, out2_bs, st);
+        return build_parents_launch<T, VEC>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, st);
+    return build_parents_launch<T, 1>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, st);
+}
+
+int build_parents_strided(const void *qp, const void *kp, const void *vp, const void *kc, const void *vc,
+                          void *out, void *out2, void *weights, int B, int P, int H, int D,
+                          const LevelStrides &in, int dtype, hipStream_t st) {
+    // zero = dense: rows H*D apart, batches rows * row stride apart
+    LevelStrides sd = in;
+    for (int i = 0; i < 7; ++i) {
+        const int64_t rows = (i == 3 || i == 4) ? 2 * (int64_t)P : (int64_t)P;
+        if (!sd.rs[i]) sd.rs[i] = (int64_t)H * D;
+        if (sd.rs[i] < (int64_t)H * D) return fail(HSA_ERR_INVALID, "row stride %lld below H*D", (long long)sd.rs[i]);
+        if (!sd.bs[i]) sd.bs[i] = rows * sd.rs[i];
+    }
+    switch (dtype) {
+        case HSA_F32: return build_parents_typed<F32>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, st);
+        case HSA_F16: return build_parents_typed<F16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, st);
+        case HSA_BF16: return build_parents_typed<BF16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, st);
+    }
+    return fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
 int build_parents_dispatch(const void *qp, const void *kp, const void *vp, const void *kc, const void *vc,
                            void *out, void *out2, void *weights, int B, int P, int H, int D, int64_t qp_bs,
                            int64_t kp_bs, int64_t vp_bs, int64_t kc_bs, int64_t vc_bs, int64_t out_bs,
                            int64_t out2_bs, int dtype, hipStream_t st) {
-    const int64_t prow = (int64_t)P * H * D, crow = 2 * prow;
-    if (!qp_bs) qp_bs = prow;
-    if (!kp_bs) kp_bs = prow;
-    if (!vp_bs) vp_bs = prow;
-    if (!out_bs) out_bs = prow;
-    if (!out2_bs) out2_bs = prow;
-    if (!kc_bs) kc_bs = crow;
-    if (!vc_bs) vc_bs = crow;
-    switch (dtype) {
-        case HSA_F32: return build_parents_typed<F32>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
-        case HSA_F16: return build_parents_typed<F16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
-        case HSA_BF16: return build_parents_typed<BF16>(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs, st);
-    }
-    return fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+    LevelStrides sd = {{qp_bs, kp_bs, vp_bs, kc_bs, vc_bs, out_bs, out2_bs}, {0, 0, 0, 0, 0, 0, 0}};
+    return build_parents_strided(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, dtype, st);
 }
 
 }  // namespace hsa
@@ -553,6 +562,22 @@ int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const 
     HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
     return hsa::build_parents_dispatch(qp, kp, vp, kc, vc, out, nullptr, weights, B, P, H, D, qp_bs, kp_bs,
                                        vp_bs, kc_bs, vc_bs, out_bs, 0, dtype, (hipStream_t)stream);
+}
+
+int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp, const void *kc,
+                                  const void *vc, void *out, void *out2, int B, int P, int H, int D,
+                                  const int64_t *batch_strides, const int64_t *row_strides, int dtype,
+                                  void *stream) {
+    HSA_REQUIRE(qp && kp && vp && kc && vc && out, "null pointer");
+    HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
+    hsa::LevelStrides sd = {};
+    for (int i = 0; i < 7; ++i) {
+        if (batch_strides) sd.bs[i] = batch_strides[i];
+        if (row_strides) sd.rs[i] = row_strides[i];
+        HSA_REQUIRE(sd.bs[i] >= 0 && sd.rs[i] >= 0, "negative stride");
+    }
+    return hsa::build_parents_strided(qp, kp, vp, kc, vc, out, out2, nullptr, B, P, H, D, sd, dtype,
+                                      (hipStream_t)stream);
 }
 
 int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const void *k_leaf,

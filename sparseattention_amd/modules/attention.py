@@ -7,13 +7,16 @@ the span attention are the HIP kernels.
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import List, Optional
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
-from ..ops.functional import build_parent_nodes, build_parents_forward, hierarchical_attention
+from .. import _lib
+from ..ops.functional import build_parent_nodes, hierarchical_attention
 from ..ops.topology import build_tree_topology
 
 
@@ -48,6 +51,7 @@ class HierarchicalAttention(nn.Module):
         self.cached_is_causal = None
         self.sizes: Optional[List[int]] = None
         self.offsets: Optional[List[int]] = None
+        self._fused = {}  # row-concatenated projection weights of the no-autograd path
 
     # -- helpers -------------------------------------------------------------
     def _get_lookup_table(self, L: int, is_causal: bool, device: torch.device):
@@ -68,6 +72,51 @@ class HierarchicalAttention(nn.Module):
     def _heads(self, t: torch.Tensor) -> torch.Tensor:
         return t.view(t.shape[0], -1, self.num_heads, self.head_dim)
 
+    def _fused_weight(self, name: str, layers) -> torch.Tensor:
+        """Weights of several bias-free projections stacked along the output dimension, so one
+        GEMM computes them all; rebuilt when any of them has been written to or moved."""
+        key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype) for m in layers)
+        hit = self._fused.get(name)
+        if hit is None or hit[0] != key:
+            hit = (key, torch.cat([m.weight.detach() for m in layers], dim=0))
+            self._fused[name] = hit
+        return hit[1]
+
+    def _cross_update_Y_direct(self, x: torch.Tensor, y_in: torch.Tensor) -> torch.Tensor:
+        """cross_update_Y without autograd and without dropout: the three projections of the span
+        nodes are one GEMM, the key/value projections of each level's children another, and each
+        level's kernel reads its operands as column slices of those results.  Every level writes
+        twice: a dense [B, P, D] block that feeds the next level's GEMM, and its slice of the
+        level-concatenated [B, N-1, D] result."""
+        B, N, D = x.shape
+        H, Dh = self.num_heads, self.head_dim
+        _lib.require_gpu(x, y_in)
+        x, y_in = x.contiguous(), y_in.contiguous()
+        qkv = F.linear(y_in, self._fused_weight("qkv_y", (self.Wq_y, self.Wk_y, self.Wv_y)))  # [B, N-1, 3D]
+        w_kv = self._fused_weight("kv_y", (self.Wk_y, self.Wv_y))
+        y_new = torch.empty((B, N - 1, D), dtype=x.dtype, device=x.device)
+        blocks = torch.empty(B * (N - 1) * D, dtype=x.dtype, device=x.device)  # level-major
+        # the level loop works on raw addresses: the operands are fixed column slices of qkv and
+        # of each level's k/v projection, so no tensor views are made per level
+        es = x.element_size()
+        A = ctypes.c_int64 * 7
+        row_strides = A(3 * D, 3 * D, 3 * D, 2 * D, 2 * D, D, D)
+        fwd, code, stream = _lib.lib().hsa_build_parents_strided_fwd, _lib.dtype_code(x), _lib.stream_of(x)
+        qkv_p, blk_p, out_p = qkv.data_ptr(), blocks.data_ptr(), y_new.data_ptr()
+        src, off = x, 0
+        with torch.cuda.device(x.device):
+            for P in self.sizes:
+                kv = F.linear(src, w_kv)  # [B, 2P, 2D]
+                par, kv_p, lvl_p = qkv_p + off * 3 * D * es, kv.data_ptr(), blk_p + B * off * D * es
+                rc = fwd(par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es, lvl_p,
+                         out_p + off * D * es, B, P, H, Dh,
+                         A((N - 1) * 3 * D, (N - 1) * 3 * D, (N - 1) * 3 * D, 4 * P * D, 4 * P * D, P * D,
+                           (N - 1) * D), row_strides, code, stream)
+                _lib.check(rc, "hsa_build_parents_strided_fwd")
+                src = blocks[B * off * D:B * (off + P) * D].view(B, P, D)
+                off += P
+        return self.out_proj_y(y_new)
+
     # -- bottom-up: leaves -> span nodes ----------------------------------------
     def cross_update_Y(self, x: torch.Tensor, y_in: torch.Tensor) -> torch.Tensor:
         B, N, D = x.shape
@@ -77,31 +126,23 @@ class HierarchicalAttention(nn.Module):
         if self.sizes is None or self.sizes[0] != N // 2:
             self.sizes, self.offsets = self._build_level_info(N)
 
+        grad = torch.is_grad_enabled() and (x.requires_grad or y_in.requires_grad
+                                            or self.Wq_y.weight.requires_grad)
+        if not grad and not (self.training and self.dropout.p > 0):
+            return self._cross_update_Y_direct(x, y_in)
+
         q_lv = torch.split(self._heads(self.Wq_y(y_in)), self.sizes, dim=1)
         k_lv = torch.split(self._heads(self.Wk_y(y_in)), self.sizes, dim=1)
         v_lv = torch.split(self._heads(self.Wv_y(y_in)), self.sizes, dim=1)
-
-        # Without autograd the level outputs go straight into one [B, N-1, D] buffer (no
-        # concatenation afterwards); with autograd each level is a differentiable op.
-        direct = not (torch.is_grad_enabled() and (x.requires_grad or y_in.requires_grad
-                                                    or self.Wq_y.weight.requires_grad))
-        y_new = torch.empty((B, N - 1, D), dtype=x.dtype, device=x.device) if direct else None
-        levels, src, off = [], x, 0
+        levels, src = [], x
         for lvl, P in enumerate(self.sizes):
             k_c = self._heads(self.Wk_y(src))
             v_c = self.dropout(self._heads(self.Wv_y(src)))
             if lvl == 0:
                 v_c = self.dropout(v_c)  # the leaf values pass through dropout twice
-            if direct:
-                dst = y_new[:, off:off + P]
-                build_parents_forward(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c,
-                                      out=dst.view(B, P, self.num_heads, self.head_dim))
-                src = dst
-            else:
-                src = build_parent_nodes(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c).reshape(B, P, D)
-                levels.append(src)
-            off += P
-        return self.out_proj_y(y_new if direct else torch.cat(levels, dim=1))
+            src = build_parent_nodes(q_lv[lvl], k_lv[lvl], v_lv[lvl], k_c, v_c).reshape(B, P, D)
+            levels.append(src)
+        return self.out_proj_y(torch.cat(levels, dim=1))
 
     # -- top-down: span nodes -> leaves -------------------------------------------
     def update_X_from_Y(self, x: torch.Tensor, y: torch.Tensor,

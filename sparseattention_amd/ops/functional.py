@@ -6,6 +6,7 @@ torch and enqueues a kernel of libhsa_gfx950.so on the current stream.
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -98,7 +99,7 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
 
 def _rows_dense(t: torch.Tensor) -> bool:
     B, rows, H, D = t.shape
-    return t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D
+    return t.stride(3) == 1 and t.stride(2) == D and (rows == 1 or t.stride(1) == H * D)
 
 
 def _batch_stride(t: torch.Tensor) -> int:
@@ -139,6 +140,34 @@ def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False,
             _lib.stream_of(Q_p))
     _lib.check(rc, "hsa_build_parents_fwd")
     return (out, weights) if return_weights else out
+
+
+def build_parents_strided(Q_p, K_p, V_p, K_c, V_c, out: torch.Tensor,
+                          out2: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One level of the parent build on operands that are column slices of wider matrices
+    (thirds of a fused q/k/v projection, halves of a fused k/v projection): each [B, rows, H, D]
+    view needs dense heads (strides D, 1) only; row and batch strides are free.  The result goes
+    to `out` and, if given, to `out2` as well.  No autograd."""
+    ts = (Q_p, K_p, V_p, K_c, V_c, out) + ((out2,) if out2 is not None else ())
+    _lib.require_gpu(*ts)
+    B, P, H, D = Q_p.shape
+    assert K_c.shape == (B, 2 * P, H, D) and V_c.shape == K_c.shape, "Child count mismatch"
+    assert K_p.shape == Q_p.shape and V_p.shape == Q_p.shape and out.shape == Q_p.shape
+    assert out2 is None or out2.shape == Q_p.shape
+    bs, rs = [0] * 7, [0] * 7
+    for i, t in enumerate(ts):
+        assert t.dtype == Q_p.dtype, "dtype mismatch"
+        assert t.stride(3) == 1 and t.stride(2) == D and t.stride(1) >= H * D, \
+            "heads of every operand must be dense"
+        rs[i] = t.stride(1)
+        bs[i] = t.stride(0) if B > 1 else t.shape[1] * t.stride(1)
+    A = ctypes.c_int64 * 7
+    with torch.cuda.device(Q_p.device):
+        rc = _lib.lib().hsa_build_parents_strided_fwd(
+            _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
+            _lib.ptr(out2), B, P, H, D, A(*bs), A(*rs), _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
+    _lib.check(rc, "hsa_build_parents_strided_fwd")
+    return out
 
 
 def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None,

@@ -148,6 +148,29 @@ def test_build_parents_vs_oracle(shape, dtype):
     assert torch.equal(out, out2)
 
 
+@pytest.mark.parametrize("shape", [(2, 5, 3, 16), (3, 32, 8, 64), (1, 1, 2, 128), (2, 7, 2, 20)])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_build_parents_column_slices(shape, dtype):
+    """Operands that are thirds / halves of wider matrices (fused projections): same bits as the
+    dense call, both outputs written, bytes around the outputs untouched."""
+    B, P, H, D = shape
+    g = torch.Generator().manual_seed(P + D)
+    qkv = torch.randn(B, P, 3, H, D, generator=g).to(dtype).to(DEV)
+    kv = torch.randn(B, 2 * P, 2, H, D, generator=g).to(dtype).to(DEV)
+    big = torch.full((B, P + 3, H, D), 7.0, dtype=dtype, device=DEV)
+    out = torch.empty(B, P, H, D, dtype=dtype, device=DEV)
+    got = fn.build_parents_strided(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], kv[:, :, 0], kv[:, :, 1],
+                                   out=out, out2=big[:, 2:2 + P])
+    ops = [t.contiguous() for t in (qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], kv[:, :, 0], kv[:, :, 1])]
+    dense = fn.build_parents_forward(*ops)
+    assert got is out and torch.equal(out, dense) and torch.equal(big[:, 2:2 + P], dense)
+    assert (big[:, :2] == 7).all() and (big[:, 2 + P:] == 7).all()
+    want = oracle.build_parent_nodes_ref(*(t.cpu() for t in ops), compute_dtype=torch.float64)
+    assert_close(out, want, dtype, "bpn column slices")
+    with pytest.raises(AssertionError):
+        fn.build_parents_strided(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], kv[:, :P, 0], kv[:, :P, 1], out=out)
+
+
 def test_build_parents_child_count_assert():
     z = torch.zeros(1, 4, 1, 8, device=DEV)
     with pytest.raises(AssertionError):
@@ -214,6 +237,28 @@ def test_module_vs_oracle(dtype, causal):
     assert (y_new.double().cpu() - want_y).abs().max() < atol
     assert (out.double().cpu() - want).abs().max() < atol
     assert md(xd, xd, xd, y=yd, mask=mask, return_attention=True)[1] is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_module_fused_projection_path_matches_level_by_level_path(dtype):
+    """Without autograd the span-node update runs on fused projections; with autograd it runs one
+    projection and one differentiable op per level.  Same result."""
+    B, N, dim, H = 2, 128, 64, 4
+    torch.manual_seed(1)
+    m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=4).to(DEV).to(dtype).eval()
+    x = torch.randn(B, N, dim, device=DEV).clamp(-1, 1).to(dtype)
+    y = torch.randn(B, N - 1, dim, device=DEV).clamp(-1, 1).to(dtype)
+    with torch.no_grad():
+        fused = m.cross_update_Y(x, y)
+        again = m.cross_update_Y(x, y)      # cached stacked weights
+        with torch.no_grad():
+            m.Wk_y.weight.mul_(1.0)           # a write invalidates the cache, values unchanged
+        third = m.cross_update_Y(x, y)
+    stepwise = m.cross_update_Y(x.requires_grad_(True), y)
+    assert stepwise.requires_grad and not fused.requires_grad
+    assert torch.equal(fused, again) and torch.equal(fused, third)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (fused.float() - stepwise.detach().float()).abs().max() < tol
 
 
 # ---------------------------------------------------------------- the configurations of the benchmark
