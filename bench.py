@@ -91,8 +91,9 @@ def lm_forward_bench(args):
     model = model.to(dev).to(torch.bfloat16).eval()
     tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(0)).to(dev)
     K = min(args.steps, 20)
+    W = max(10, min(args.warmup, 20))  # the first forwards also grow the allocator's pools
     with torch.no_grad():
-        for _ in range(3):
+        for _ in range(W):
             model(tok)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -124,7 +125,7 @@ def lm_forward_bench(args):
     share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
-        "value": B * N / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": 3,
+        "value": B * N / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "cfg4: decoder LM forward, random init, eval mode"},

@@ -112,6 +112,35 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
                                   int dtype, void *stream);
 
 /*
+ * The last levels of HierarchicalAttention.cross_update_Y in one launch
+ * (hierarchical_attention/modules/attention.py:119-157: per level the children's
+ * Wk_y / Wv_y projections :141-142, build_parent_nodes :145-153, the output feeding the next
+ * level :157).  16-bit element types.  Starting from C rows `src` (the output of the level
+ * below, or the leaves of a short sequence), every remaining level up to the root is computed
+ * on chip: projection by MFMA, rounded to the element type like a separate GEMM's output, then
+ * the 3-way softmax per parent and head.
+ *
+ *   src    [B, C, H*Dh]      dense rows; C a power of two, 2 <= C <= hsa_cross_update_top_rows
+ *   qkv    parents' q | k | v rows ([.., 3*H*Dh] per row), pointing at the first parent of the
+ *          first level computed here; the C-1 parents follow level after level, root last
+ *   w_kv   the Wk_y / Wv_y weights in the kernel's operand order, 2*(H*Dh)^2 elements,
+ *          written by hsa_cross_update_pack_weights from the two [H*Dh, H*Dh] row-major
+ *          weight matrices (row = output feature); repack after the weights change
+ *   out    result rows, numbered like qkv's, H*Dh elements each
+ *   *_bs, *_rs  batch / row strides in elements (0 = dense)
+ *
+ * hsa_cross_update_top_rows returns the largest C the kernel holds for this head layout
+ * (0 = not handled: fp32, or a head size other than 32 / 64 / 128, or H*Dh not a multiple of
+ * 128); hsa_cross_update_top_fwd returns HSA_ERR_UNSUPPORTED for such shapes.
+ */
+int hsa_cross_update_top_rows(int H, int Dh, int dtype);
+int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh,
+                                  int dtype, void *stream);
+int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv, void *out, int B,
+                             int C, int H, int Dh, int64_t src_bs, int64_t qkv_bs, int64_t qkv_rs,
+                             int64_t out_bs, int64_t out_rs, int dtype, void *stream);
+
+/*
  * Whole tree in one call: level 1 from the leaves, every further level from the
  * previous level's output used as both child K and child V (the composition
  * Out_l = build_parent_nodes(Qp_l, Kp_l, Vp_l, Out_{l-1}, Out_{l-1}) of the op at

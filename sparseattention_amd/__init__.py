@@ -4,6 +4,7 @@ Exports the reference library's public names (hierarchical_attention/__init__.py
 """
 __version__ = "0.1.0"
 
+from ._lib import HsaError  # noqa: F401,E402
 from .modules import HierarchicalAttention  # noqa: F401,E402
 from .ops import (  # noqa: F401,E402
     attention_forward,
@@ -25,5 +26,6 @@ __all__ = [
     "hierarchical_attention",
     "build_tree",
     "attention_forward",
+    "HsaError",
     "__version__",
 ]

@@ -38,6 +38,12 @@ def _declare(lib):
     lib.hsa_build_parents_fwd.restype = I
     lib.hsa_build_parents_strided_fwd.argtypes = [P] * 7 + [I] * 4 + [P, P, I, P]
     lib.hsa_build_parents_strided_fwd.restype = I
+    lib.hsa_cross_update_top_rows.argtypes = [I, I, I]
+    lib.hsa_cross_update_top_rows.restype = I
+    lib.hsa_cross_update_pack_weights.argtypes = [P, P, P, I, I, I, P]
+    lib.hsa_cross_update_pack_weights.restype = I
+    lib.hsa_cross_update_top_fwd.argtypes = [P] * 4 + [I] * 4 + [I64] * 5 + [I, P]
+    lib.hsa_cross_update_top_fwd.restype = I
     lib.hsa_build_tree_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 7 + [I, P]
     lib.hsa_build_tree_fwd.restype = I
     lib.hsa_topology_host.argtypes = [I, I, P, P, P]

@@ -33,61 +33,11 @@
 #pragma once
 
 #include "hsa_common.h"
+#include "hsa_mma.h"
 
 #include <type_traits>
 
 namespace hsa {
-
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef short s16x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-
-template <typename T> struct Mma;
-
-template <> struct Mma<BF16> {
-    static constexpr uint16_t kOne = 0x3f80;
-    static __device__ __forceinline__ f32x4 k32(u32x4_t a, u32x4_t b, f32x4 c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ f32x4 k16(u32x2_t a, u32x2_t b, f32x4 c) {
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
-                                                         __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
-    }
-    // round-to-nearest-even pair
-    static __device__ __forceinline__ uint32_t pack(float a, float b) {
-        f32x2 v = {a, b};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-    }
-    // the inputs are exactly representable: keep the high halves
-    static __device__ __forceinline__ uint32_t pack_exact(float a, float b) {
-        return (__float_as_uint(a) >> 16) | (__float_as_uint(b) & 0xffff0000u);
-    }
-};
-
-template <> struct Mma<F16> {
-    static constexpr uint16_t kOne = 0x3c00;
-    static __device__ __forceinline__ f32x4 k32(u32x4_t a, u32x4_t b, f32x4 c) {
-        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a),
-                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ f32x4 k16(u32x2_t a, u32x2_t b, f32x4 c) {
-        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a),
-                                                     __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ uint32_t pack(float a, float b) {
-        f32x2 v = {a, b};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
-    }
-    static __device__ __forceinline__ uint32_t pack_exact(float a, float b) { return pack(a, b); }
-};
 
 constexpr int TILE_Q = 16;           // queries per block
 constexpr int TILE_MAX_SB = 4;        // a strip is at most 64 aligned queries

@@ -39,30 +39,6 @@ __device__ __forceinline__ void store_vec(typename T::storage *p, const float (&
     }
 }
 
-// 3-way softmax with the reference kernel's epsilon in the denominator.  fp32 tensors get
-// the accurate exp and division; 16-bit tensors (output precision 2^-9 or 2^-11) use the
-// hardware exp2 and reciprocal.
-template <typename T>
-__device__ __forceinline__ void softmax3(float s0, float s1, float s2, float &w0, float &w1, float &w2) {
-    float m = fmaxf(s0, fmaxf(s1, s2));
-    if constexpr (sizeof(typename T::storage) == 4) {
-        float e0 = expf(s0 - m), e1 = expf(s1 - m), e2 = expf(s2 - m);
-        float den = e0 + e1 + e2 + 1e-9f;
-        w0 = e0 / den;
-        w1 = e1 / den;
-        w2 = e2 / den;
-    } else {
-        constexpr float kLog2e = 1.4426950408889634f;
-        float e0 = __builtin_amdgcn_exp2f((s0 - m) * kLog2e);
-        float e1 = __builtin_amdgcn_exp2f((s1 - m) * kLog2e);
-        float e2 = __builtin_amdgcn_exp2f((s2 - m) * kLog2e);
-        float inv = __builtin_amdgcn_rcpf(e0 + e1 + e2 + 1e-9f);
-        w0 = e0 * inv;
-        w1 = e1 * inv;
-        w2 = e2 * inv;
-    }
-}
-
 // Batch and row strides (in elements) of the seven operands of one level, in the order
 // qp, kp, vp, kc, vc, out, out2.  A row stride wider than H*D reads a column slice of a
 // wider matrix, e.g. one third of a fused q/k/v projection.

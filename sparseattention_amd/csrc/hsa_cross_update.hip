@@ -1,0 +1,366 @@
+// Upper levels of the span-node update in one launch (16-bit element types).
+//
+// In the module each level l of the bottom-up pass is
+//     [k_c | v_c] = src_l * W_kv^T              (projection of the children, all heads)
+//     out_l       = parent build(q_l, k_l, v_l, k_c, v_c)     (3-way softmax per parent and head)
+//     src_{l+1}   = out_l
+// Near the root a level is a few rows, so a launch per projection and per parent build costs
+// far more than the work.  Here one workgroup per batch element walks the last levels: the
+// level's rows live in LDS, a wavefront owns a head, multiplies the rows by the head's 2*Dh
+// weight rows with MFMA (weights streamed from L2 in a pre-packed operand order, so that every
+// load instruction of a wavefront reads 1 KiB of consecutive bytes; the rows read from LDS),
+// rounds the result to
+// the element type as the separate projection would, and finishes the parent build from the
+// accumulator registers: in the MFMA result layout a lane holds four consecutive rows of one
+// column, i.e. both children of two parents, so the three scores need only a sum over the 16
+// lanes that share those rows.  The level's output goes to the result tensor and to the other
+// LDS buffer, which is the next level's input.
+#include "hsa_mma.h"
+
+#include <atomic>
+
+namespace hsa {
+
+namespace {
+
+constexpr int TOP_WAVES = 8;      // two per SIMD: up to 256 VGPRs each
+constexpr int TOP_LDS_MAX = 160 * 1024;
+
+struct TopParams {
+    const uint16_t *src;  // [B, C0, Dm]  children of the first level handled here, dense rows
+    const uint16_t *qkv;  // parents' q | k | v: row j of this pointer = j-th parent handled here
+    const uint16_t *w;    // packed key / value projection weights (see pack_kv_kernel)
+    uint16_t *out;        // result rows, numbered like qkv's
+    int64_t src_bs, qkv_bs, qkv_rs, out_bs, out_rs;
+    int B, H, Dm, C0;
+    float scale;
+};
+
+template <typename T> __device__ __forceinline__ float rounded(float x) {
+    return to_float<T>(from_float<T>(x));
+}
+
+// One level: C children in `cur` (LDS, 16*RT rows readable), C/2 parents out.  Two passes per
+// head over the level's rows: the key columns give the softmax weights, the value columns the
+// output, so only Dh accumulator columns are live at a time.
+template <typename T, int CT2, int RT>
+__device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int row, const unsigned char *cur,
+                                          unsigned char *nxt, int pitch) {
+    using M_ = Mma<T>;
+    constexpr int Dh = 16 * CT2;
+    constexpr int PD = CT2 >= 8 ? 2 : 4;    // weight k-steps in flight
+    constexpr bool EARLY = RT * CT2 <= 8;   // registers allow the parents' rows to be requested before the projection
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r16 = lane & 15, g = lane >> 4;
+    const int Dm = p.Dm, NK = Dm / 32, P = C >> 1;
+    const unsigned char *arow = cur + r16 * pitch + 16 * g;
+
+    for (int h = wave; h < p.H; h += TOP_WAVES) {
+        // parent e of row tile rt in this lane: 8rt + 2g + e, children = accumulator rows 2e, 2e+1
+        const uint16_t *prow[RT][2];
+        bool valid[RT][2];
+        int prel[RT][2];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int pe = 8 * rt + 2 * g + e;
+                valid[rt][e] = pe < P;
+                prel[rt][e] = valid[rt][e] ? pe : P - 1;
+                prow[rt][e] = p.qkv + (size_t)b * p.qkv_bs + (size_t)(row + prel[rt][e]) * p.qkv_rs + h * Dh + r16;
+            }
+
+        // acc[rt][ct] = rows 16rt.. of `cur` times weight rows wbase + 16ct + (0..15):
+        // lane (r16, g) ends with column r16 of tile ct, rows 16rt + 4g .. +3.
+        // The weights of PD k-steps are in flight while one step is multiplied; the scheduling
+        // barriers keep the compiler from sinking those loads down to their first use.
+        f32x4 acc[RT][CT2];
+        auto project = [&](int half) {
+            // packed weights: [half][head][k-step][column tile][lane][8 elements]
+            const uint16_t *wp = p.w + ((size_t)(half * p.H + h) * NK * CT2 * 64 + lane) * 8;
+            const unsigned char *ap = arow;
+            u32x4_t bq[PD][CT2];
+            auto load_b = [&](int u, int kofs) {
+#pragma unroll
+                for (int ct = 0; ct < CT2; ++ct)
+                    bq[u][ct] = *reinterpret_cast<const u32x4_t *>(wp + (kofs * CT2 + ct) * 512);
+            };
+            auto step = [&](int u, bool prefetch) {
+                u32x4_t a[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    a[rt] = *reinterpret_cast<const u32x4_t *>(ap + 16 * rt * pitch + 64 * u);
+#pragma unroll
+                for (int ct = 0; ct < CT2; ++ct)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = M_::k32(a[rt], bq[u][ct], acc[rt][ct]);
+                if (prefetch) load_b(u, u + PD);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int ct = 0; ct < CT2; ++ct) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < PD; ++u) load_b(u, u);  // NK >= PD (Dm is a multiple of 128)
+            __builtin_amdgcn_sched_barrier(0);
+            for (int ks0 = 0; ks0 + PD < NK; ks0 += PD) {
+#pragma unroll
+                for (int u = 0; u < PD; ++u) step(u, true);
+                wp += PD * CT2 * 512;
+                ap += 64 * PD;
+            }
+#pragma unroll
+            for (int u = 0; u < PD; ++u) step(u, false);
+        };
+
+        // ---- keys: the three scores and the softmax weights ----
+        uint16_t rq[RT][2][CT2], rk[RT][2][CT2];
+        auto load_qk = [&]() {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+#pragma unroll
+                    for (int c = 0; c < CT2; ++c) {
+                        rq[rt][e][c] = prow[rt][e][16 * c];
+                        rk[rt][e][c] = prow[rt][e][Dm + 16 * c];
+                    }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if (EARLY) load_qk();
+        project(0);
+        if (!EARLY) load_qk();
+        float wgt[RT][2][3];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int c = 0; c < CT2; ++c) {
+                    const float fq = to_float<T>(rq[rt][e][c]);
+                    s0 = fmaf(fq, to_float<T>(rk[rt][e][c]), s0);
+                    s1 = fmaf(fq, rounded<T>(acc[rt][c][2 * e]), s1);
+                    s2 = fmaf(fq, rounded<T>(acc[rt][c][2 * e + 1]), s2);
+                }
+                s0 = group_sum(s0, 16);
+                s1 = group_sum(s1, 16);
+                s2 = group_sum(s2, 16);
+                softmax3<T>(s0 * p.scale, s1 * p.scale, s2 * p.scale, wgt[rt][e][0], wgt[rt][e][1], wgt[rt][e][2]);
+            }
+        }
+
+        // ---- values: the weighted sum, to the result tensor and to the next level's rows ----
+        uint16_t rv[RT][2][CT2];
+        auto load_v = [&]() {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int e = 0; e < 2; ++e)
+#pragma unroll
+                    for (int c = 0; c < CT2; ++c) rv[rt][e][c] = prow[rt][e][2 * Dm + 16 * c];
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if (EARLY) load_v();
+        project(1);
+        if (!EARLY) load_v();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                uint16_t *orow = p.out + (size_t)b * p.out_bs + (size_t)(row + prel[rt][e]) * p.out_rs + h * Dh + r16;
+                uint16_t *lrow = reinterpret_cast<uint16_t *>(nxt + prel[rt][e] * pitch) + h * Dh + r16;
+#pragma unroll
+                for (int c = 0; c < CT2; ++c) {
+                    const float o = wgt[rt][e][0] * to_float<T>(rv[rt][e][c]) +
+                                    wgt[rt][e][1] * rounded<T>(acc[rt][c][2 * e]) +
+                                    wgt[rt][e][2] * rounded<T>(acc[rt][c][2 * e + 1]);
+                    const uint16_t r = from_float<T>(o);
+                    if (valid[rt][e]) {
+                        orow[16 * c] = r;
+                        lrow[16 * c] = r;
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T, int CT2, int RT0>
+__global__ void __launch_bounds__(TOP_WAVES * 64) cross_update_top_kernel(TopParams p) {
+    extern __shared__ __align__(16) unsigned char top_smem[];
+    const int b = blockIdx.x;
+    const int Dm = p.Dm;
+    const int pitch = Dm * 2 + 16;
+    unsigned char *buf0 = top_smem;
+    unsigned char *buf1 = top_smem + 16 * RT0 * pitch;
+    {
+        const int cpr = Dm / 8;  // 16-byte pieces per row
+        const uint16_t *src = p.src + (size_t)b * p.src_bs;
+        for (int i = threadIdx.x; i < p.C0 * cpr; i += TOP_WAVES * 64) {
+            const int r = i / cpr, c = i - r * cpr;
+            *reinterpret_cast<u32x4_t *>(buf0 + r * pitch + 16 * c) =
+                *reinterpret_cast<const u32x4_t *>(src + (size_t)r * Dm + 8 * c);
+        }
+    }
+    __syncthreads();
+    int C = p.C0, row = 0;
+    unsigned char *cur = buf0, *nxt = buf1;
+    auto advance = [&]() {
+        __syncthreads();
+        row += C >> 1;
+        C >>= 1;
+        unsigned char *t = cur;
+        cur = nxt;
+        nxt = t;
+    };
+    if constexpr (RT0 >= 4) {
+        top_level<T, CT2, 4>(p, b, C, row, cur, nxt, pitch);
+        advance();
+    }
+    if constexpr (RT0 >= 2) {
+        top_level<T, CT2, 2>(p, b, C, row, cur, nxt, pitch);
+        advance();
+    }
+    while (C >= 2) {
+        top_level<T, CT2, 1>(p, b, C, row, cur, nxt, pitch);
+        advance();
+    }
+}
+
+// Weights into MFMA operand order: packed[half][h][ks][ct][lane = 16g + r][0..7] =
+// W_half[h*Dh + 16ct + r][32ks + 8g + 0..7], half 0 = keys, 1 = values.  One thread per
+// 16-byte piece.
+__global__ void __launch_bounds__(256) pack_kv_kernel(const uint16_t *__restrict__ wk, const uint16_t *__restrict__ wv,
+                                                      uint16_t *__restrict__ packed, int H, int Dh, int Dm) {
+    const int CT2 = Dh / 16, NK = Dm / 32;
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= 2L * Dm * Dm / 8) return;
+    const int lane = (int)(idx & 63);
+    long t = idx >> 6;
+    const int ct = (int)(t % CT2); t /= CT2;
+    const int ks = (int)(t % NK); t /= NK;
+    const int h = (int)(t % H);
+    const int half = (int)(t / H);
+    const int r = lane & 15, g = lane >> 4;
+    const uint16_t *src = (half ? wv : wk) + (size_t)(h * Dh + 16 * ct + r) * Dm + 32 * ks + 8 * g;
+    *reinterpret_cast<u32x4_t *>(packed + idx * 8) = *reinterpret_cast<const u32x4_t *>(src);
+}
+
+// row tiles the first level may have: registers first, then LDS
+int top_row_tiles(int H, int Dh) {
+    int rt = 16 / (Dh / 16);  // RT * (Dh/16) accumulator tiles <= 16
+    if (rt > 4) rt = 4;
+    const long pitch = (long)H * Dh * 2 + 16;
+    while (rt >= 1 && (16L * rt + (rt >= 2 ? 8L * rt : 16L)) * pitch > TOP_LDS_MAX) rt >>= 1;
+    return rt;
+}
+
+bool top_shape_ok(int H, int Dh, int dtype) {
+    if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
+    if (Dh != 32 && Dh != 64 && Dh != 128) return false;
+    if (H < 1 || ((long)H * Dh) % 128 != 0) return false;
+    return top_row_tiles(H, Dh) >= 1;
+}
+
+template <typename T, int CT2, int RT0>
+int top_launch_rt(const TopParams &p, hipStream_t st) {
+    const int pitch = p.Dm * 2 + 16;
+    const size_t lds = (size_t)(16 * RT0 + (RT0 >= 2 ? 8 * RT0 : 16)) * pitch;
+    auto kern = cross_update_top_kernel<T, CT2, RT0>;
+    if (lds > 64 * 1024) {
+        // raising the limit is slow: once per kernel and device, for the largest size it is asked for
+        static std::atomic<size_t> allowed[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(HSA_ERR_LAUNCH, "no current device");
+        if (allowed[dev].load(std::memory_order_acquire) < lds) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "LDS size %zu refused: %s", lds, hipGetErrorString(e));
+            allowed[dev].store(lds, std::memory_order_release);
+        }
+    }
+    kern<<<p.B, TOP_WAVES * 64, lds, st>>>(p);
+    return check_launch("cross_update_top_kernel");
+}
+
+template <typename T, int CT2>
+int top_launch_ct(const TopParams &p, hipStream_t st) {
+    const int rt0 = p.C0 >= 64 ? 4 : (p.C0 >= 32 ? 2 : 1);
+    if constexpr (CT2 <= 4) {
+        if (rt0 == 4) return top_launch_rt<T, CT2, 4>(p, st);
+    }
+    if (rt0 == 2) return top_launch_rt<T, CT2, 2>(p, st);
+    if (rt0 == 1) return top_launch_rt<T, CT2, 1>(p, st);
+    return fail(HSA_ERR_UNSUPPORTED, "too many rows (%d) for head_dim %d", p.C0, 16 * CT2);
+}
+
+template <typename T>
+int top_launch(const TopParams &p, int Dh, hipStream_t st) {
+    switch (Dh) {
+        case 32: return top_launch_ct<T, 2>(p, st);
+        case 64: return top_launch_ct<T, 4>(p, st);
+        case 128: return top_launch_ct<T, 8>(p, st);
+    }
+    return fail(HSA_ERR_UNSUPPORTED, "head_dim %d", Dh);
+}
+
+}  // namespace
+
+}  // namespace hsa
+
+extern "C" {
+
+int hsa_cross_update_top_rows(int H, int Dh, int dtype) {
+    if (!hsa::top_shape_ok(H, Dh, dtype)) return 0;
+    return 16 * hsa::top_row_tiles(H, Dh);
+}
+
+int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh, int dtype,
+                                  void *stream) {
+    HSA_REQUIRE(wk && wv && packed, "null pointer");
+    if (!hsa::top_shape_ok(H, Dh, dtype))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "shape H=%d Dh=%d dtype=%d not handled by the fused levels", H, Dh, dtype);
+    HSA_REQUIRE((((uintptr_t)wk | (uintptr_t)wv | (uintptr_t)packed) & 15) == 0, "weights must be 16-byte aligned");
+    const int Dm = H * Dh;
+    const long pieces = 2L * Dm * Dm / 8;
+    hsa::pack_kv_kernel<<<(unsigned)((pieces + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t *)wk, (const uint16_t *)wv, (uint16_t *)packed, H, Dh, Dm);
+    return hsa::check_launch("pack_kv_kernel");
+}
+
+int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv, void *out, int B, int C,
+                             int H, int Dh, int64_t src_bs, int64_t qkv_bs, int64_t qkv_rs, int64_t out_bs,
+                             int64_t out_rs, int dtype, void *stream) {
+    HSA_REQUIRE(src && qkv && w_kv && out, "null pointer");
+    HSA_REQUIRE(B >= 1 && H >= 1 && Dh >= 1, "bad shape B=%d H=%d Dh=%d", B, H, Dh);
+    HSA_REQUIRE(C >= 2 && hsa::ilog2_exact(C) >= 0, "row count must be a power of two >= 2 (got %d)", C);
+    if (!hsa::top_shape_ok(H, Dh, dtype))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "shape H=%d Dh=%d dtype=%d not handled by the fused levels", H, Dh, dtype);
+    if (C > 16 * hsa::top_row_tiles(H, Dh))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "%d rows exceed the %d the fused levels hold", C,
+                         16 * hsa::top_row_tiles(H, Dh));
+    const int64_t Dm = (int64_t)H * Dh;
+    if (!src_bs) src_bs = (int64_t)C * Dm;
+    if (!qkv_rs) qkv_rs = 3 * Dm;
+    if (!out_rs) out_rs = Dm;
+    if (!qkv_bs) qkv_bs = (int64_t)(C - 1) * qkv_rs;
+    if (!out_bs) out_bs = (int64_t)(C - 1) * out_rs;
+    HSA_REQUIRE(qkv_rs >= 3 * Dm && out_rs >= Dm, "row strides below the row length");
+    HSA_REQUIRE((((uintptr_t)src | (uintptr_t)w_kv) & 15) == 0 && src_bs % 8 == 0,
+                "src and w_kv must be 16-byte aligned");
+    hsa::TopParams p;
+    p.src = (const uint16_t *)src;
+    p.qkv = (const uint16_t *)qkv;
+    p.w = (const uint16_t *)w_kv;
+    p.out = (uint16_t *)out;
+    p.src_bs = src_bs; p.qkv_bs = qkv_bs; p.qkv_rs = qkv_rs; p.out_bs = out_bs; p.out_rs = out_rs;
+    p.B = B; p.H = H; p.Dm = (int)Dm; p.C0 = C;
+    p.scale = 1.0f / sqrtf((float)Dh);
+    if (dtype == HSA_BF16) return hsa::top_launch<hsa::BF16>(p, Dh, (hipStream_t)stream);
+    return hsa::top_launch<hsa::F16>(p, Dh, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -16,7 +16,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .. import _lib
-from ..ops.functional import build_parent_nodes, hierarchical_attention
+from ..ops.functional import build_parent_nodes, hierarchical_attention, pack_kv_weights
 from ..ops.topology import build_tree_topology
 
 
@@ -52,6 +52,7 @@ class HierarchicalAttention(nn.Module):
         self.sizes: Optional[List[int]] = None
         self.offsets: Optional[List[int]] = None
         self._fused = {}  # row-concatenated projection weights of the no-autograd path
+        self.fuse_top_levels = True  # no-autograd path: the last levels in one launch where the shape allows
 
     # -- helpers -------------------------------------------------------------
     def _get_lookup_table(self, L: int, is_causal: bool, device: torch.device):
@@ -72,13 +73,15 @@ class HierarchicalAttention(nn.Module):
     def _heads(self, t: torch.Tensor) -> torch.Tensor:
         return t.view(t.shape[0], -1, self.num_heads, self.head_dim)
 
-    def _fused_weight(self, name: str, layers) -> torch.Tensor:
+    def _fused_weight(self, name: str, layers, packed: bool = False) -> torch.Tensor:
         """Weights of several bias-free projections stacked along the output dimension, so one
-        GEMM computes them all; rebuilt when any of them has been written to or moved."""
+        GEMM computes them all (packed: key / value weights in the operand order of the fused
+        upper levels); rebuilt when any of them has been written to or moved."""
         key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype) for m in layers)
         hit = self._fused.get(name)
         if hit is None or hit[0] != key:
-            hit = (key, torch.cat([m.weight.detach() for m in layers], dim=0))
+            ws = [m.weight.detach() for m in layers]
+            hit = (key, pack_kv_weights(ws[0], ws[1], self.num_heads) if packed else torch.cat(ws, dim=0))
             self._fused[name] = hit
         return hit[1]
 
@@ -87,7 +90,8 @@ class HierarchicalAttention(nn.Module):
         nodes are one GEMM, the key/value projections of each level's children another, and each
         level's kernel reads its operands as column slices of those results.  Every level writes
         twice: a dense [B, P, D] block that feeds the next level's GEMM, and its slice of the
-        level-concatenated [B, N-1, D] result."""
+        level-concatenated [B, N-1, D] result.  The last levels (few rows each) run as one
+        launch that does their projections on chip."""
         B, N, D = x.shape
         H, Dh = self.num_heads, self.head_dim
         _lib.require_gpu(x, y_in)
@@ -103,9 +107,19 @@ class HierarchicalAttention(nn.Module):
         row_strides = A(3 * D, 3 * D, 3 * D, 2 * D, 2 * D, D, D)
         fwd, code, stream = _lib.lib().hsa_build_parents_strided_fwd, _lib.dtype_code(x), _lib.stream_of(x)
         qkv_p, blk_p, out_p = qkv.data_ptr(), blocks.data_ptr(), y_new.data_ptr()
+        # child rows the fused upper levels take (0: shape not handled)
+        top_rows = _lib.lib().hsa_cross_update_top_rows(H, Dh, code) if self.fuse_top_levels else 0
         src, off = x, 0
         with torch.cuda.device(x.device):
             for P in self.sizes:
+                if 2 * P <= top_rows:
+                    # the remaining levels fit one workgroup per batch: a single launch
+                    w_top = self._fused_weight("kv_y_packed", (self.Wk_y, self.Wv_y), packed=True)
+                    rc = _lib.lib().hsa_cross_update_top_fwd(
+                        src.data_ptr(), qkv_p + off * 3 * D * es, w_top.data_ptr(), out_p + off * D * es,
+                        B, 2 * P, H, Dh, 0, (N - 1) * 3 * D, 3 * D, (N - 1) * D, D, code, stream)
+                    _lib.check(rc, "hsa_cross_update_top_fwd")
+                    break
                 kv = F.linear(src, w_kv)  # [B, 2P, 2D]
                 par, kv_p, lvl_p = qkv_p + off * 3 * D * es, kv.data_ptr(), blk_p + B * off * D * es
                 rc = fwd(par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es, lvl_p,

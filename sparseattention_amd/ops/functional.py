@@ -170,6 +170,56 @@ def build_parents_strided(Q_p, K_p, V_p, K_c, V_c, out: torch.Tensor,
     return out
 
 
+def fused_top_rows(num_heads: int, head_dim: int, dtype: torch.dtype) -> int:
+    """Largest number of child rows `cross_update_top` takes for this head layout (0: the
+    layout is not handled and every level has to go through `build_parents_strided`)."""
+    if dtype not in (torch.float16, torch.bfloat16):
+        return 0
+    code = 1 if dtype == torch.float16 else 2
+    return int(_lib.lib().hsa_cross_update_top_rows(num_heads, head_dim, code))
+
+
+def pack_kv_weights(w_k: torch.Tensor, w_v: torch.Tensor, num_heads: int) -> torch.Tensor:
+    """Key and value projection weights ([dim, dim] each, row = output feature) in the operand
+    order `cross_update_top` streams them in.  Repack whenever the weights change."""
+    _lib.require_gpu(w_k, w_v)
+    dim = w_k.shape[0]
+    assert w_k.shape == (dim, dim) and w_v.shape == (dim, dim) and w_k.dtype == w_v.dtype
+    w_k, w_v = w_k.contiguous(), w_v.contiguous()
+    packed = torch.empty(2 * dim * dim, dtype=w_k.dtype, device=w_k.device)
+    with torch.cuda.device(w_k.device):
+        rc = _lib.lib().hsa_cross_update_pack_weights(
+            _lib.ptr(w_k), _lib.ptr(w_v), _lib.ptr(packed), num_heads, dim // num_heads,
+            _lib.dtype_code(w_k), _lib.stream_of(w_k))
+    _lib.check(rc, "hsa_cross_update_pack_weights")
+    return packed
+
+
+def cross_update_top(src: torch.Tensor, qkv: torch.Tensor, w_packed: torch.Tensor, out: torch.Tensor,
+                     num_heads: int) -> torch.Tensor:
+    """Every level from `src` up to the root in one launch: per level the children are projected
+    with the key / value weights (`w_packed` from `pack_kv_weights`), the parents are built, and
+    the parents are the next level's children.
+
+    src [B, C, dim] dense; qkv [B, C-1, 3*dim] the parents' q | k | v, level after level, root
+    last; out [B, C-1, dim] numbered alike.  qkv and out may be row slices of larger tensors."""
+    _lib.require_gpu(src, qkv, w_packed, out)
+    B, C, dim = src.shape
+    H, Dh = num_heads, dim // num_heads
+    assert src.is_contiguous() and w_packed.is_contiguous() and w_packed.numel() == 2 * dim * dim
+    assert qkv.shape == (B, C - 1, 3 * dim) and out.shape == (B, C - 1, dim)
+    assert qkv.stride(2) == 1 and out.stride(2) == 1
+    assert src.dtype == qkv.dtype == w_packed.dtype == out.dtype, "dtype mismatch"
+    with torch.cuda.device(src.device):
+        rc = _lib.lib().hsa_cross_update_top_fwd(
+            _lib.ptr(src), _lib.ptr(qkv), _lib.ptr(w_packed), _lib.ptr(out), B, C, H, Dh, 0,
+            qkv.stride(0) if B > 1 else 0, qkv.stride(1) if C > 2 else 0,
+            out.stride(0) if B > 1 else 0, out.stride(1) if C > 2 else 0,
+            _lib.dtype_code(src), _lib.stream_of(src))
+    _lib.check(rc, "hsa_cross_update_top_fwd")
+    return out
+
+
 def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None,
                out2: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Every tree level in one call: level 1 from the leaves, level l+1 from level l's

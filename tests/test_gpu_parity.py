@@ -171,6 +171,59 @@ def test_build_parents_column_slices(shape, dtype):
         fn.build_parents_strided(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], kv[:, :P, 0], kv[:, :P, 1], out=out)
 
 
+@pytest.mark.parametrize("B,C,H,Dh", [(2, 64, 8, 64), (3, 32, 4, 32), (1, 2, 2, 64), (2, 16, 2, 128), (2, 32, 4, 128),
+                                      (1, 8, 16, 32), (2, 64, 12, 32)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cross_update_top_levels(B, C, H, Dh, dtype):
+    """All levels above C rows in one launch: against the mathematics in fp64 (projection, 3-way
+    softmax, level after level) and against the level-by-level kernels."""
+    dim = H * Dh
+    assert C <= fn.fused_top_rows(H, Dh, dtype)
+    g = torch.Generator().manual_seed(C + H)
+    src = torch.randn(B, C, dim, generator=g).clamp(-1, 1).to(dtype)
+    big = torch.randn(B, C + 4, 3 * dim, generator=g).clamp(-1, 1).to(dtype)   # parents' rows sit at 3..C+1
+    w = (torch.randn(2 * dim, dim, generator=g) / dim ** 0.5).to(dtype)
+    qkv = big[:, 3:3 + C - 1]
+    outbig = torch.full((B, C + 1, dim), 5.0, dtype=dtype, device=DEV)
+    bigd = big.to(DEV)
+    wp = fn.pack_kv_weights(w[:dim].to(DEV), w[dim:].to(DEV), H)
+    got = fn.cross_update_top(src.to(DEV), bigd[:, 3:3 + C - 1], wp, outbig[:, 1:C], H)
+    assert (outbig[:, 0] == 5).all() and (outbig[:, C] == 5).all()
+    # fp64 on the same 16-bit inputs
+    cur, off, P, want = src.double(), 0, C // 2, []
+    while P >= 1:
+        kv = torch.nn.functional.linear(cur, w.double()).view(B, 2 * P, 2, H, Dh)
+        par = qkv[:, off:off + P].double().view(B, P, 3, H, Dh)
+        o = oracle.build_parent_nodes_ref(par[:, :, 0], par[:, :, 1], par[:, :, 2], kv[:, :, 0], kv[:, :, 1])
+        cur = o.reshape(B, P, dim)
+        want.append(cur)
+        off, P = off + P, P // 2
+    want = torch.cat(want, dim=1)
+    assert (got.double().cpu() - want).abs().max() < 3e-2
+    # level by level on the GPU (each level's projection rounded to the element type, as here)
+    cur, off, P, ref = src.to(DEV), 0, C // 2, []
+    while P >= 1:
+        kv = torch.nn.functional.linear(cur, w.to(DEV)).view(B, 2 * P, 2, H, Dh)
+        par = bigd[:, 3 + off:3 + off + P].view(B, P, 3, H, Dh)
+        o = torch.empty(B, P, H, Dh, dtype=dtype, device=DEV)
+        fn.build_parents_strided(par[:, :, 0], par[:, :, 1], par[:, :, 2], kv[:, :, 0], kv[:, :, 1], out=o)
+        cur = o.view(B, P, dim)
+        ref.append(cur)
+        off, P = off + P, P // 2
+    assert (got.float() - torch.cat(ref, dim=1).float()).abs().max() < 2e-2
+
+
+def test_cross_update_top_shapes_not_handled():
+    assert fn.fused_top_rows(8, 64, torch.float32) == 0
+    assert fn.fused_top_rows(3, 24, torch.bfloat16) == 0
+    assert fn.fused_top_rows(8, 64, torch.bfloat16) == 64 and fn.fused_top_rows(8, 128, torch.bfloat16) == 32
+    z = torch.zeros(1, 128, 512, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(sa.HsaError):
+        fn.cross_update_top(z, torch.zeros(1, 127, 1536, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(1024 * 512, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(1, 127, 512, dtype=torch.bfloat16, device=DEV), 8)
+
+
 def test_build_parents_child_count_assert():
     z = torch.zeros(1, 4, 1, 8, device=DEV)
     with pytest.raises(AssertionError):
