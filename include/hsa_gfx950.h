@@ -71,6 +71,21 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
                  int D, int L, int R, int causal, int dtype, int algo, void *stream);
 
+/*
+ * hsa_attn_fwd that also reports the kernel's own execution interval: `start_event` and
+ * `stop_event` (hipEvent_t, created by the caller with timing enabled) are attached to the
+ * span-attention dispatch and carry the kernel's begin and end timestamps, so
+ * hipEventElapsedTime(start, stop) is the kernel duration without the idle gap between
+ * consecutive launches that events recorded around a call include.  (The gather kernels record
+ * the events around the launch instead.)  The reference times its kernels with torch events
+ * around the Python call (hierarchical_attention_project/Hierarchical_Attention_Triton_Test.py
+ * :523-568); this is the same measurement taken at the dispatch.
+ */
+int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_t *idx,
+                       const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
+                       int D, int L, int R, int causal, int dtype, int algo, void *stream,
+                       void *start_event, void *stop_event);
+
 /* 1 if HSA_ATTN_AUTO would pick the MFMA tile kernel for this problem, else 0. */
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype,
                            int canonical_tables, int want_weights);

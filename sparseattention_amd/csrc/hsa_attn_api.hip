@@ -45,8 +45,24 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
                          N, H, D, L, R, dtype, (int)canonical);
     if (tile_ok && algo != HSA_ATTN_GATHER)
         return hsa::attn_tile_dispatch(q, k, v, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0, dtype, st);
-    return hsa::attn_gather_dispatch(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0,
-                                     dtype, st);
+    // the gather kernels take no dispatch events: record around the call instead
+    const hsa::LaunchEvents ev = hsa::take_launch_events();
+    if (ev.start && ev.stop) (void)hipEventRecord(ev.start, st);
+    const int rc = hsa::attn_gather_dispatch(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R,
+                                             causal ? 1 : 0, dtype, st);
+    if (ev.start && ev.stop) (void)hipEventRecord(ev.stop, st);
+    return rc;
+}
+
+int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_t *idx,
+                       const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H, int D,
+                       int L, int R, int causal, int dtype, int algo, void *stream, void *start_event,
+                       void *stop_event) {
+    HSA_REQUIRE(start_event && stop_event, "null event");
+    hsa::set_launch_events((hipEvent_t)start_event, (hipEvent_t)stop_event);
+    const int rc = hsa_attn_fwd(q, k, v, idx, mask, out, weights, B, N, M, H, D, L, R, causal, dtype, algo, stream);
+    (void)hsa::take_launch_events();  // an argument error returns before any launcher looks
+    return rc;
 }
 
 }  // extern "C"

@@ -3,13 +3,20 @@
 #pragma once
 #include "hsa_attn_tile.h"
 
+#include <hip/hip_ext.h>
+
 namespace hsa {
 
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
 static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
     if (wpb > tile_max_wpb<D>()) wpb = tile_max_wpb<D>();
     const int nwg = (p.n_units + wpb - 1) / wpb;
-    attn_tile_kernel<T, D, NBW, CAUSAL, SB><<<nwg, wpb * 64, 0, st>>>(p);
+    const LaunchEvents ev = take_launch_events();
+    if (ev.start && ev.stop)
+        hipExtLaunchKernelGGL((attn_tile_kernel<T, D, NBW, CAUSAL, SB>), dim3(nwg), dim3(wpb * 64), 0, st, ev.start,
+                              ev.stop, 0, p);
+    else
+        attn_tile_kernel<T, D, NBW, CAUSAL, SB><<<nwg, wpb * 64, 0, st>>>(p);
     return check_launch("attn_tile_kernel");
 }
 

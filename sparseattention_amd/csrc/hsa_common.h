@@ -15,6 +15,15 @@ void set_error(const char *fmt, ...);
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
 
+// ---- optional timing of the next kernel launch of this host thread -----------------------------
+// hsa_attn_fwd_timed leaves a pair of events here; the launcher that finds them attaches them
+// to the kernel dispatch itself (recorded at the kernel's begin and end) and clears the slot.
+struct LaunchEvents {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+void set_launch_events(hipEvent_t start, hipEvent_t stop);
+LaunchEvents take_launch_events();
+
 #define HSA_REQUIRE(cond, ...)                                    \
     do {                                                          \
         if (!(cond)) return ::hsa::fail(HSA_ERR_INVALID, __VA_ARGS__); \

@@ -23,6 +23,17 @@ int fail(int code, const char *fmt, ...) {
     return code;
 }
 
+static thread_local LaunchEvents g_launch_events;
+void set_launch_events(hipEvent_t start, hipEvent_t stop) {
+    g_launch_events.start = start;
+    g_launch_events.stop = stop;
+}
+LaunchEvents take_launch_events() {
+    LaunchEvents e = g_launch_events;
+    g_launch_events = LaunchEvents();
+    return e;
+}
+
 int check_launch(const char *what) {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));

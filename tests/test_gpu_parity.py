@@ -129,6 +129,38 @@ def test_attention_inputs_untouched_and_noncontiguous():
     assert_close(out, want, torch.float32)
 
 
+def test_timed_entry_point_same_output_and_a_kernel_interval():
+    """hsa_attn_fwd_timed: identical result, and the two events bracket the kernel itself."""
+    import ctypes
+    from sparseattention_amd import _lib
+    B, N, H, D, R = 2, 256, 4, 64, 8
+    L, M = 8, 2 * N - 1
+    q, k, v = make_qkv(B, N, H, D, torch.bfloat16, seed=3)
+    qd, kd, vd = q.to(DEV), k.to(DEV), v.to(DEV)
+    t = sa.build_tree_topology(N, True, device=DEV)
+    want = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R)
+    lib = _lib.lib()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(); e1.record()          # creates the underlying HIP events
+    torch.cuda.synchronize()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    for algo in (_lib.ATTN_TILE, _lib.ATTN_GATHER):
+        out = torch.zeros_like(qd)
+        rc = lib.hsa_attn_fwd_timed(_lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd), None, None, _lib.ptr(out), None,
+                                    B, N, M, H, D, L, R, 1, _lib.HSA_BF16, algo, st,
+                                    ctypes.c_void_p(e0.cuda_event), ctypes.c_void_p(e1.cuda_event))
+        assert rc == 0, lib.hsa_last_error()
+        torch.cuda.synchronize()
+        ref = want if algo == _lib.ATTN_TILE else fn.attention_forward(qd, kd, vd, t["forward_idx"],
+                                                                       t["forward_mask"], R, algo="gather")
+        assert torch.equal(out, ref)
+        assert 0.0 < e0.elapsed_time(e1) < 50.0
+    # a plain call afterwards is not affected by the events of the timed one
+    assert torch.equal(fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R), want)
+    assert lib.hsa_attn_fwd_timed(_lib.ptr(qd), _lib.ptr(kd), _lib.ptr(vd), None, None, _lib.ptr(out), None,
+                                  B, N, M, H, D, L, R, 1, _lib.HSA_BF16, 0, st, None, None) == -22
+
+
 # ---------------------------------------------------------------- parent build
 @pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20),
                                    (3, 33, 12, 64)])
