@@ -319,12 +319,14 @@ static int build_subtree_launch(const void *qp, const void *kp, const void *vp, 
 constexpr int TOP_MAX_LEVELS = 8;
 constexpr int TOP_THREADS = 1024;
 
-template <typename T, int VEC>
+// GT: lanes per parent row when known at compile time (the reductions then need no branches), 0 = use G
+template <typename T, int VEC, int GT>
 __global__ void __launch_bounds__(TOP_THREADS)
 build_top_kernel(const typename T::storage *__restrict__ Qp, const typename T::storage *__restrict__ Kp,
                  const typename T::storage *__restrict__ Vp, typename T::storage *__restrict__ Out,
                  typename T::storage *__restrict__ Out2, int N, int H, int D, int G, int lvl0, int nlev,
                  int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t out_bs, int64_t out2_bs, float scale) {
+    if (GT) G = GT;
     using S = typename T::storage;
     using P = Pack<T, VEC>;
     extern __shared__ __align__(16) unsigned char top_lds[];
@@ -385,9 +387,9 @@ build_top_kernel(const typename T::storage *__restrict__ Qp, const typename T::s
                     s1 = fmaf(q, to_float<T>(c0.e[e]), s1);
                     s2 = fmaf(q, to_float<T>(c1.e[e]), s2);
                 }
-                s0 = group_sum(s0, G);
-                s1 = group_sum(s1, G);
-                s2 = group_sum(s2, G);
+                s0 = group_sum(s0, GT ? GT : G);
+                s1 = group_sum(s1, GT ? GT : G);
+                s2 = group_sum(s2, GT ? GT : G);
                 float w0, w1, w2;
                 softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
                 P r;
@@ -424,9 +426,14 @@ static int build_top_launch(const void *qp, const void *kp, const void *vp, void
     const float scale = 1.0f / sqrtf((float)D);
     int threads = (nc / 2) * G;
     if (threads < 64) threads = 64;
-    build_top_kernel<T, VEC><<<B * H, threads, lds, st>>>((const S *)qp, (const S *)kp, (const S *)vp, (S *)out,
-                                                          (S *)out2, N, H, D, G, lvl0, nlev, qp_bs, kp_bs, vp_bs,
-                                                          out_bs, out2_bs, scale);
+#define HSA_TOP_LAUNCH(GT)                                                                              \
+    build_top_kernel<T, VEC, GT><<<B * H, threads, lds, st>>>((const S *)qp, (const S *)kp, (const S *)vp, \
+                                                              (S *)out, (S *)out2, N, H, D, G, lvl0, nlev, \
+                                                              qp_bs, kp_bs, vp_bs, out_bs, out2_bs, scale)
+    if (G == 8) HSA_TOP_LAUNCH(8);
+    else if (G == 16) HSA_TOP_LAUNCH(16);
+    else HSA_TOP_LAUNCH(0);
+#undef HSA_TOP_LAUNCH
     return check_launch("build_top_kernel");
 }
 
