@@ -163,10 +163,23 @@ class HierarchicalAttention(nn.Module):
                         mask: Optional[torch.Tensor] = None) -> torch.Tensor:
         B, N, D = x.shape
         assert y is not None, "y (parents) cannot be None during top-down update"
-        xy = torch.cat([x, y], dim=1)
         q = self._heads(self.Wq_x(x))
-        k = self._heads(self.Wk_x(xy))
-        v = self.dropout(self._heads(self.Wv_x(xy)))
+        grad = torch.is_grad_enabled() and (x.requires_grad or y.requires_grad
+                                            or self.Wk_x.weight.requires_grad)
+        if not grad and not (self.training and self.dropout.p > 0) and y.size(1) == N - 1:
+            # leaves and span nodes are projected straight into their rows of the [B, 2N-1, D]
+            # key / value buffers (batched GEMMs with a strided output): no concatenated input
+            k = torch.empty((B, 2 * N - 1, D), dtype=x.dtype, device=x.device)
+            v = torch.empty_like(k)
+            for lin, dst in ((self.Wk_x, k), (self.Wv_x, v)):
+                wt = lin.weight.t().unsqueeze(0).expand(B, D, D)
+                torch.bmm(x, wt, out=dst[:, :N])
+                torch.bmm(y, wt, out=dst[:, N:])
+            k, v = self._heads(k), self._heads(v)
+        else:
+            xy = torch.cat([x, y], dim=1)
+            k = self._heads(self.Wk_x(xy))
+            v = self.dropout(self._heads(self.Wv_x(xy)))
         is_causal = mask is not None  # only the presence of a mask is looked at
         t = self._get_lookup_table(N, is_causal, x.device)
         heads = hierarchical_attention(q, k, v, t["forward_idx"], t["backward_gather"],
