@@ -78,6 +78,8 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
         assert out.shape == Q.shape and out.dtype == Q.dtype and out.is_contiguous() and out.is_cuda
     weights = (torch.empty((B, N, H, 2 * R + 1 + L), device=Q.device, dtype=torch.float32)
                if return_weights else None)
+    if Q.numel() == 0:  # empty batch: nothing to launch
+        return (out, weights) if return_weights else out
     lib = _lib.lib()
     with torch.cuda.device(Q.device):
         if canon is not None and M >= 2 * N - 1:
@@ -132,6 +134,8 @@ def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False,
     else:
         assert out.shape == (B, P, H, D) and out.dtype == Q_p.dtype and _rows_dense(out)
     weights = torch.empty((B, P, H, 3), device=Q_p.device, dtype=Q_p.dtype) if return_weights else None
+    if Q_p.numel() == 0:
+        return (out, weights) if return_weights else out
     with torch.cuda.device(Q_p.device):
         rc = _lib.lib().hsa_build_parents_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
@@ -240,6 +244,8 @@ def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None
     assert out.shape == Q_p.shape and out.dtype == Q_p.dtype
     if out2 is not None:
         assert out2.shape == Q_p.shape and out2.dtype == Q_p.dtype
+    if K_leaf.numel() == 0:
+        return out
     ts = [Q_p, K_p, V_p, K_leaf, V_leaf]
     for i, t in enumerate(ts):
         if not (t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D):
@@ -262,6 +268,8 @@ def build_parents_backward(grad_out, Q_p, K_p, V_p, K_c, V_c):
     B, P, H, D = Q_p.shape
     dq, dkp, dvp = torch.empty_like(Q_p), torch.empty_like(K_p), torch.empty_like(V_p)
     dkc, dvc = torch.empty_like(K_c), torch.empty_like(V_c)
+    if Q_p.numel() == 0:
+        return dq, dkp, dvp, dkc, dvc
     with torch.cuda.device(Q_p.device):
         rc = _lib.lib().hsa_build_parents_bwd(
             _lib.ptr(grad_out), _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c),
@@ -280,6 +288,8 @@ def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool, algo: 
     L = N.bit_length() - 1
     R = int(window_size)
     dq, dk, dv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    if Q.numel() == 0:
+        return dq, dk, dv
     lib = _lib.lib()
     nbytes = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(Q), _lib.algo_code(algo)))
     ws = torch.empty((max(nbytes, 4) + 3) // 4, device=Q.device, dtype=torch.float32)

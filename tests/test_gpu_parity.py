@@ -161,6 +161,21 @@ def test_timed_entry_point_same_output_and_a_kernel_interval():
                                   B, N, M, H, D, L, R, 1, _lib.HSA_BF16, 0, st, None, None) == -22
 
 
+def test_empty_batch_gives_empty_outputs():
+    N, H, D = 16, 2, 8
+    t = sa.build_tree_topology(N, True, device=DEV)
+    z = lambda rows: torch.zeros(0, rows, H, D, device=DEV, requires_grad=True)
+    q, k, v = z(N), z(2 * N - 1), z(2 * N - 1)
+    out = sa.hierarchical_attention(q, k, v, t["forward_idx"], t["backward_gather"], t["forward_mask"], 2)
+    assert out.shape == (0, N, H, D)
+    out.sum().backward()
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape
+    par = sa.build_parent_nodes(z(4), z(4), z(4), z(8), z(8))
+    assert par.shape == (0, 4, H, D)
+    par.sum().backward()
+    assert sa.build_tree(z(N - 1), z(N - 1), z(N - 1), z(N), z(N)).shape == (0, N - 1, H, D)
+
+
 # ---------------------------------------------------------------- parent build
 @pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20),
                                    (3, 33, 12, 64)])
