@@ -197,12 +197,16 @@ __global__ void __launch_bounds__(TOP_WAVES * 64) cross_update_top_kernel(TopPar
     unsigned char *buf0 = top_smem;
     unsigned char *buf1 = top_smem + 16 * RT0 * pitch;
     {
-        const int cpr = Dm / 8;  // 16-byte pieces per row
+        // The MFMA passes always read whole 16-row tiles: rows that hold no node (fewer than 16
+        // children in a level) are zero, never uninitialised memory.
+        constexpr int ROWS = 16 * RT0 + (RT0 >= 2 ? 8 * RT0 : 16);
+        const int cpr = (Dm + 8) / 8;  // 16-byte pieces per padded row
         const uint16_t *src = p.src + (size_t)b * p.src_bs;
-        for (int i = threadIdx.x; i < p.C0 * cpr; i += TOP_WAVES * 64) {
+        for (int i = threadIdx.x; i < ROWS * cpr; i += TOP_WAVES * 64) {
             const int r = i / cpr, c = i - r * cpr;
-            *reinterpret_cast<u32x4_t *>(buf0 + r * pitch + 16 * c) =
-                *reinterpret_cast<const u32x4_t *>(src + (size_t)r * Dm + 8 * c);
+            u32x4_t val = {0u, 0u, 0u, 0u};
+            if (r < p.C0 && 8 * c < Dm) val = *reinterpret_cast<const u32x4_t *>(src + (size_t)r * Dm + 8 * c);
+            *reinterpret_cast<u32x4_t *>(top_smem + r * pitch + 16 * c) = val;
         }
     }
     __syncthreads();
