@@ -405,11 +405,15 @@ TILE_CASES = [  # B, N, H, D, R
 @pytest.mark.parametrize("case", TILE_CASES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("strip", [None, "1", "3"])
+@pytest.mark.parametrize("strip", [None, "1", "2", "4", "4-same-direction"])
 def test_attention_tile_vs_oracle(case, dtype, causal, strip, monkeypatch):
+    """Strip length forced to 1 / 2 / 4 query blocks (longer strips alternate their walking
+    direction between neighbours unless told otherwise) and the dispatcher's own choice."""
     B, N, H, D, R = case
     if strip is not None:
-        monkeypatch.setenv("HSA_ATTN_TILE_SB", strip)
+        monkeypatch.setenv("HSA_ATTN_TILE_SB", strip[0])
+        if strip.endswith("same-direction"):
+            monkeypatch.setenv("HSA_ATTN_TILE_ALT", "0")
     q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
     t = sa.build_tree_topology(N, causal, device=DEV)
     o = oracle.topology_tables(N, causal)
