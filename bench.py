@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--noncausal", action="store_true")
     ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
+    ap.add_argument("--streams", type=int, default=2,
+                    help="HIP streams the steps alternate between (each step is an independent batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -159,6 +161,17 @@ def main():
     set_bytes = e * B * H * D * (N + 2 * M + N + 3 * (N - 1))
     nsets = args.sets or max(3, -(-512 * 2**20 // set_bytes))
 
+    stream = torch.cuda.current_stream(dev)
+    st = ctypes.c_void_p(stream.cuda_stream)
+    # Steps are independent batches: they alternate between `--streams` HIP streams (default
+    # priority), so one step's short-of-work kernels (the top of the tree runs on 64 of 256 CUs)
+    # overlap the next step's streaming kernels.  A buffer set always goes to the same stream, so
+    # two steps that touch the same buffers are ordered.
+    nstreams = max(1, args.streams)
+    while nsets % nstreams:
+        nsets += 1
+    side = [torch.cuda.Stream(device=dev) for _ in range(nstreams)] if nstreams > 1 else [stream]
+    side_st = [ctypes.c_void_p(x.cuda_stream) for x in side]
     g = torch.Generator().manual_seed(0)
     sets = []
     for _ in range(nsets):
@@ -170,24 +183,25 @@ def main():
         s["kfull"][:, :N] = mk(N)
         s["vfull"][:, :N] = mk(N)
         sets.append(s)
+    torch.cuda.synchronize()  # the inputs were written on the current stream
 
-    stream = torch.cuda.current_stream(dev)
-    st = ctypes.c_void_p(stream.cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     node_off = N * H * D * e
     full_bs = M * H * D
 
-    def tree_args(s):
+    def tree_args(s, st):
         return (P(s["qp"]), P(s["kp"]), P(s["vp"]), P(s["kfull"]), P(s["vfull"]),
                 ctypes.c_void_p(s["kfull"].data_ptr() + node_off), ctypes.c_void_p(s["vfull"].data_ptr() + node_off),
                 B, N, H, D, 0, 0, 0, full_bs, full_bs, full_bs, full_bs, _lib.HSA_BF16, st)
 
-    def attn_args(s):
+    def attn_args(s, st):
         return (P(s["q"]), P(s["kfull"]), P(s["vfull"]), None, None, P(s["out"]), None,
                 B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st)
 
-    targs = [tree_args(s) for s in sets]
-    aargs = [attn_args(s) for s in sets]
+    targs = [tree_args(s, st) for s in sets]          # everything on the current stream
+    aargs = [attn_args(s, st) for s in sets]
+    targs_p = [tree_args(s, side_st[i % nstreams]) for i, s in enumerate(sets)]   # set i on stream i % nstreams
+    aargs_p = [attn_args(s, side_st[i % nstreams]) for i, s in enumerate(sets)]
     assert lib.hsa_attn_fwd_uses_tile(N, M, H, D, L, R, _lib.HSA_BF16, 1, 0) == 1
 
     # HIP events whose timestamps are the attention kernel's own begin and end (attached to the
@@ -216,8 +230,13 @@ def main():
             rc |= lib.hsa_attn_fwd_timed(*aargs[i % nsets], ev[0], ev[1])
         return rc
 
+    def step_p(i):
+        rc = lib.hsa_build_tree_fwd(*targs_p[i % nsets])
+        rc |= lib.hsa_attn_fwd(*aargs_p[i % nsets])
+        return rc
+
     for i in range(args.warmup):
-        assert step(i) == 0, lib.hsa_last_error()
+        assert step_p(i) == 0, lib.hsa_last_error()
     torch.cuda.synchronize()
 
     # --- timed region: exactly K steps between two synchronisations -----------------------
@@ -226,11 +245,22 @@ def main():
     t0 = time.perf_counter()
     rc = 0
     for i in range(K):
-        rc |= step(i)
+        rc |= step_p(i)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     assert rc == 0, lib.hsa_last_error()
     ms_per_step = (t1 - t0) * 1e3 / K
+
+    # --- the same K steps one after the other on a single stream (the latency of a step) ----
+    for i in range(min(args.warmup, 10)):
+        rc |= step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        rc |= step(i)
+    torch.cuda.synchronize()
+    serial_ms_per_step = (time.perf_counter() - t0) * 1e3 / K
+    assert rc == 0, lib.hsa_last_error()
 
     # --- duration of the dominant kernel: the same K steps once more, every attention dispatch
     #     carrying its own pair of HIP events (kept out of the region above because an
@@ -310,16 +340,18 @@ def main():
         "n_gpus": 1, "steps": K, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "%s: %s; step = tree build + span attention forward" % (args.workload, desc),
+        "config": {"workload": "%s: %s; step = tree build + span attention forward on one batch; independent batches alternate between %d HIP streams" % (args.workload, desc, nstreams),
                    "B": B, "H": H, "N": N, "D": D, "window_radius": R, "causal": causal,
-                   "buffer_sets_rotated": nsets, "bytes_per_set": set_bytes},
+                   "buffer_sets_rotated": nsets, "bytes_per_set": set_bytes, "streams": nstreams},
         "roofline": {"bound": "hbm", "kernel": "attn_tile_kernel (span attention forward)",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_ms": attn_avg_ms,
                      "median_launch_ms": attn_kernel_ms[K // 2],
                      "timing": "HIP events attached to each attention dispatch (kernel begin/end) over a repeat of the K timed steps"},
-        "detail": {"attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
+        "detail": {"single_stream_ms_per_step": serial_ms_per_step,
+                   "single_stream_head_queries_per_s": head_queries / (serial_ms_per_step * 1e-3),
+                   "attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
                    "attn_back_to_back_ms_incl_launch_gaps": attn_b2b_ms,
                    "tree_build_avg_launch_ms": tree_b2b_ms,
                    "tree_algorithmic_bytes": tree_bytes,
