@@ -34,6 +34,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--noncausal", action="store_true")
+    ap.add_argument("--seq-len", type=int, default=0, help="override the workload's N (a power of two)")
     ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
     ap.add_argument("--streams", type=int, default=2,
                     help="HIP streams the steps alternate between (each step is an independent batch)")
@@ -151,6 +152,10 @@ def main():
     if args.workload == "cfg4":
         return lm_forward_bench(args)
     B, H, N, D, R, scale, desc = WORKLOADS[args.workload]
+    if args.seq_len:
+        assert args.seq_len >= 64 and args.seq_len & (args.seq_len - 1) == 0, "--seq-len must be a power of two >= 64"
+        desc = desc.replace("N%d" % N, "N%d" % args.seq_len)
+        N = args.seq_len
     causal = not args.noncausal
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -326,7 +331,7 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "attn_tile_%s_traffic.json" % args.workload)
     if os.path.exists(tpath):
         rec = json.load(open(tpath))
-        if rec.get("causal") == causal:
+        if rec.get("causal") == causal and not args.seq_len:
             traffic = rec["traffic_bytes_per_launch"]
 
     head_queries = B * N * H
@@ -363,7 +368,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, H, N, D, R, causal, scale, args.cpu_seconds)
-    if args.workload != "cfg3" or not causal:
+    if args.workload != "cfg3" or not causal or args.seq_len:
         result["metric"] = "attn fwd queries/sec + % HBM roofline, " + desc
     print(json.dumps(result))
 
