@@ -352,7 +352,7 @@ def main():
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_ms": attn_avg_ms,
-                     "median_launch_ms": attn_kernel_ms[K // 2],
+                     "median_launch_ms": attn_kernel_ms[K // 2], "min_launch_ms": attn_kernel_ms[0],
                      "timing": "HIP events attached to each attention dispatch (kernel begin/end) over a repeat of the K timed steps"},
         "detail": {"single_stream_ms_per_step": serial_ms_per_step,
                    "single_stream_head_queries_per_s": head_queries / (serial_ms_per_step * 1e-3),
