@@ -176,6 +176,33 @@ def test_empty_batch_gives_empty_outputs():
     assert sa.build_tree(z(N - 1), z(N - 1), z(N - 1), z(N), z(N)).shape == (0, N - 1, H, D)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_kernels_match_committed_vectors(causal):
+    """tests/golden/small_case.npz: tables bit-exact, fp32 outputs and weights within 1e-5."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small_case.npz"))
+    tag = "causal" if causal else "full"
+    t = sa.build_tree_topology(64, causal, device=DEV)
+    np.testing.assert_array_equal(t["forward_idx"].cpu().numpy(), g["idx_" + tag])
+    np.testing.assert_array_equal(t["forward_mask"].cpu().numpy(), g["mask_" + tag])
+    np.testing.assert_array_equal(t["backward_gather"].cpu().numpy(), g["gather_" + tag])
+    q, k, v = (torch.from_numpy(g[n]).to(DEV) for n in "qkv")
+    out, w = fn.attention_forward(q, k, v, t["forward_idx"], t["forward_mask"] if causal else None,
+                                  int(g["radius"]), return_weights=True)
+    assert (out.cpu() - torch.from_numpy(g["attn_out_" + tag])).abs().max() < 1e-5
+    assert (w.cpu() - torch.from_numpy(g["attn_weights_" + tag])).abs().max() < 1e-5
+    ops = [torch.from_numpy(g[n]).to(DEV) for n in ("qp", "kp", "vp", "kc", "vc")]
+    po, pw = fn.build_parents_forward(*ops, return_weights=True)
+    assert (po.cpu() - torch.from_numpy(g["parents_out"])).abs().max() < 1e-5
+    assert (pw.cpu() - torch.from_numpy(g["parents_weights"])).abs().max() < 1e-5
+    # bf16 on the same vectors, at its own tolerance
+    qb, kb, vb = (x.to(torch.bfloat16) for x in (q, k, v))
+    ob = fn.attention_forward(qb, kb, vb, t["forward_idx"], t["forward_mask"] if causal else None,
+                              int(g["radius"]))
+    ref = torch.from_numpy(g["attn_out_" + tag])
+    assert ((ob.float().cpu() - ref).abs() <= 6e-2 + 1e-2 * ref.abs()).all()   # inputs rounded to bf16 as well
+
+
 # ---------------------------------------------------------------- parent build
 @pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20),
                                    (3, 33, 12, 64)])

@@ -252,3 +252,30 @@ def test_oracle_gradients_are_true_derivatives():
     qp, kp, vp = (torch.randn(1, 2, 1, 4, generator=g, dtype=torch.float64, requires_grad=True) for _ in range(3))
     kc, vc = (torch.randn(1, 4, 1, 4, generator=g, dtype=torch.float64, requires_grad=True) for _ in range(2))
     assert torch.autograd.gradcheck(oracle.build_parent_nodes_ref, (qp, kp, vp, kc, vc), eps=1e-6, atol=1e-6)
+
+
+# ---------------------------------------------------------------- committed vectors
+def _golden():
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small_case.npz"))
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_oracle_matches_committed_vectors(causal):
+    """tests/golden/small_case.npz (written by the scalar brute force) against the torch oracle."""
+    g = _golden()
+    tag = "causal" if causal else "full"
+    t = oracle.topology_tables(64, causal)
+    np.testing.assert_array_equal(t["forward_idx"], g["idx_" + tag])
+    np.testing.assert_array_equal(t["forward_mask"], g["mask_" + tag])
+    np.testing.assert_array_equal(t["backward_gather"], g["gather_" + tag])
+    q, k, v = (torch.from_numpy(g[n]) for n in "qkv")
+    out, w = oracle.attention_ref(q, k, v, t["forward_idx"], t["forward_mask"] if causal else None,
+                                  int(g["radius"]), compute_dtype=torch.float64, return_weights=True)
+    assert (out.double() - torch.from_numpy(g["attn_out_" + tag]).double()).abs().max() < 1e-6
+    assert (w.double() - torch.from_numpy(g["attn_weights_" + tag]).double()).abs().max() < 1e-6
+    ops = [torch.from_numpy(g[n]) for n in ("qp", "kp", "vp", "kc", "vc")]
+    po, pw = oracle.build_parent_nodes_ref(*ops, compute_dtype=torch.float64, return_weights=True)
+    assert (po.double() - torch.from_numpy(g["parents_out"]).double()).abs().max() < 1e-6
+    assert (pw.double() - torch.from_numpy(g["parents_weights"]).double()).abs().max() < 1e-6
+
