@@ -78,7 +78,7 @@ attn_tile_kernel(TileParams p) {
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // leaf key blocks per query block
     constexpr int CPR = D / 8;                         // 16-byte pieces per head-row
     constexpr int RPI = 64 / CPR;                      // rows covered by one load instruction
-    constexpr int NLD = TILE_Q / RPI;                  // load instructions per 16-row block (= 2*KS)
+    constexpr int NLD = TILE_Q / RPI;                  // load instructions per 16-row block
     constexpr int PITCH = D * 2 + 16;                  // LDS row pitch in bytes (padding spreads banks)
     constexpr int BLK_BYTES = TILE_Q * PITCH;          // one 16-row operand block in LDS
     constexpr int WAVE_LDS = 5 * BLK_BYTES;            // q, k, v, near-tree k, near-tree v

@@ -12,7 +12,7 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
     (void)H;
     if (!canonical || want_weights) return false;
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
-    if (D != 64 && D != 128) return false;
+    if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS) return false;
     if (M < 2 * N - 1) return false;
     if ((R + TILE_Q - 1) / TILE_Q > TILE_MAX_NBW) return false;
@@ -49,9 +49,11 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (dtype == HSA_BF16) {
+        if (D == 32) return attn_tile_launch_td<BF16, 32>(p, nbw, causal != 0, sb, wpb, st);
         if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, sb, wpb, st);
         return attn_tile_launch_td<BF16, 128>(p, nbw, causal != 0, sb, wpb, st);
     }
+    if (D == 32) return attn_tile_launch_td<F16, 32>(p, nbw, causal != 0, sb, wpb, st);
     if (D == 64) return attn_tile_launch_td<F16, 64>(p, nbw, causal != 0, sb, wpb, st);
     return attn_tile_launch_td<F16, 128>(p, nbw, causal != 0, sb, wpb, st);
 }

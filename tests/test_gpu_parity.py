@@ -426,6 +426,9 @@ TILE_CASES = [  # B, N, H, D, R
     (1, 128, 2, 128, 32),
     (2, 64, 2, 128, 5),
     (1, 64, 2, 64, 0),
+    (2, 128, 4, 32, 8),
+    (1, 64, 3, 32, 20),
+    (1, 1024, 8, 32, 16),
 ]
 
 
