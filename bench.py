@@ -125,6 +125,29 @@ def lm_forward_bench(args):
         model(tok)
         torch.cuda.synchronize()
         cls.cross_update_Y, attn_mod.hierarchical_attention = orig_c, orig_h
+
+        # the same forward captured once into a HIP graph and replayed (no host work per launch);
+        # a replay must reproduce the eager logits bit for bit, else the figure is not reported
+        graph_ms = None
+        eager = model(tok)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model(tok)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = model(tok)
+        graph.replay()
+        torch.cuda.synchronize()
+        if torch.equal(captured, eager):
+            t0 = time.perf_counter()
+            for _ in range(K):
+                graph.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - t0) * 1e3 / K
+            if not torch.equal(captured, eager):
+                graph_ms = None
     share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
@@ -134,6 +157,7 @@ def lm_forward_bench(args):
         "config": {"workload": "cfg4: decoder LM forward, random init, eval mode"},
         "detail": {"ms_in_cross_update_Y_event_pairs": share["cross_update_Y"],
                    "ms_in_hierarchical_attention_event_pairs": share["hierarchical_attention"],
+                   "hip_graph_replay_ms_per_forward": graph_ms,
                    "calls_cross_update_Y": len(spans["cross_update_Y"]),
                    "calls_hierarchical_attention": len(spans["hierarchical_attention"])}}))
 

@@ -244,6 +244,35 @@ def test_step_replays_from_a_hip_graph():
         assert torch.equal(got, out) and torch.equal(nodes, kfull[:, N:]), "replay %d differs" % rep
 
 
+def test_lm_forward_replays_from_a_hip_graph():
+    """The whole decoder forward (projections by torch, tree and attention by the HIP kernels,
+    fused upper levels included) captured into one graph; replays on new token ids, with eager
+    forwards and synchronisations in between, equal the eager logits bit for bit."""
+    torch.manual_seed(0)
+    V, N, B = 211, 256, 2
+    model = sa.TransformerLM(V, 256, 4, 512, 2, dropout=0.0, window_size=8, activation="gelu", max_len=N)
+    model = model.to(DEV).to(torch.bfloat16).eval()
+    tok = torch.randint(0, V, (B, N), device=DEV)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                model(tok)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(tok)
+        for rep in range(3):
+            tok.copy_(torch.randint(0, V, (B, N), device=DEV))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.clone()
+            want = model(tok)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), "replay %d differs" % rep
+
+
 # ---------------------------------------------------------------- parent build
 @pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20),
                                    (3, 33, 12, 64)])
