@@ -524,6 +524,27 @@ def test_attention_tile_vs_oracle(case, dtype, causal, strip, monkeypatch):
     assert_close(out, want, dtype, "tile")
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_attention_random_shapes(seed):
+    """Seeded random shapes through whichever kernel the dispatcher picks, against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    N = int(2 ** rng.integers(1, 10))
+    D = int(rng.choice([8, 16, 20, 32, 64, 128]))
+    H = int(rng.integers(1, 6))
+    B = int(rng.integers(1, 3))
+    R = int(rng.integers(0, 40))
+    causal = bool(rng.integers(0, 2))
+    dtype = [torch.float32, torch.bfloat16, torch.float16][int(rng.integers(0, 3))]
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=seed)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    o = oracle.topology_tables(N, causal)
+    out = sa.hierarchical_attention(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], t["backward_gather"],
+                                    t["forward_mask"] if causal else None, R)
+    want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
+                                compute_dtype=torch.float64)
+    assert_close(out, want, dtype, "B%d N%d H%d D%d R%d causal=%s %s" % (B, N, H, D, R, causal, dtype))
+
+
 def test_tile_is_the_default_for_the_headline_shape():
     from sparseattention_amd import _lib
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 1, 0) == 1
