@@ -74,9 +74,41 @@ def cpu_baseline(B, H, N, D, R, causal, scale, budget_s):
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
-    return {"value": bs * N * H / med, "unit": "head-queries/s", "cores": cores, "kind": "port",
-            "sample": "%d of %d batches of the same workload (bf16, torch CPU, %d threads), median of %d passes"
-                      % (bs, B, cores, len(times))}
+    res = {"value": bs * N * H / med, "unit": "head-queries/s", "cores": cores, "kind": "port",
+           "sample": "%d of %d batches of the same workload (bf16, torch CPU, %d threads), median of %d passes"
+                     % (bs, B, cores, len(times))}
+    res["cfg1_fp32"] = cpu_plumbing_case(oracle, cores)
+    return res
+
+
+def cpu_plumbing_case(oracle, cores):
+    """The CPU-runnable configuration (B2 H4 N256 head 32, fp32, radius 8, causal and not): the CPU
+    restatement timed in full and compared with the GPU kernel on the same seeded inputs."""
+    import torch
+    from sparseattention_amd.ops import functional as fn
+    import sparseattention_amd as sa
+    B, H, N, D, R = 2, 4, 256, 32, 8
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, N, H, D, generator=g)
+    k = torch.randn(B, 2 * N - 1, H, D, generator=g)
+    v = torch.randn(B, 2 * N - 1, H, D, generator=g)
+    out = {"B": B, "H": H, "N": N, "D": D, "window_radius": R, "cores": cores}
+    for causal in (True, False):
+        t = oracle.topology_tables(N, causal)
+        m = t["forward_mask"] if causal else None
+        ts = []
+        for _ in range(7):
+            t0 = time.perf_counter()
+            want = oracle.attention_ref(q, k, v, t["forward_idx"], m, R)
+            ts.append(time.perf_counter() - t0)
+        ts = sorted(ts[2:])  # two warm-ups, median of five
+        td = sa.build_tree_topology(N, causal, device="cuda:0")
+        got = fn.attention_forward(q.cuda(), k.cuda(), v.cuda(), td["forward_idx"],
+                                   td["forward_mask"] if causal else None, R)
+        tag = "causal" if causal else "noncausal"
+        out[tag + "_cpu_head_queries_per_s"] = B * N * H / ts[len(ts) // 2]
+        out[tag + "_gpu_vs_cpu_max_abs_err"] = (got.cpu() - want).abs().max().item()
+    return out
 
 
 def lm_forward_bench(args):
