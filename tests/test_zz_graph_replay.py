@@ -1,0 +1,81 @@
+"""HIP-graph capture of the path: the entry points allocate nothing, never synchronise and launch
+on the stream they are given, so sequences of calls replay from a graph.  Collected last: these
+tests also exercise torch's own kernels under capture."""
+import pytest
+import torch
+
+import sparseattention_amd as sa
+from sparseattention_amd.ops import functional as fn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_step_replays_from_a_hip_graph():
+    """Tree build + span attention captured once into a graph (the entry points allocate nothing,
+    never synchronise and launch on the stream they are given), replayed on fresh inputs with
+    eager work and synchronisations between the replays; every replay equals the eager result."""
+    B, N, H, D, R = 2, 256, 4, 64, 16
+    g = torch.Generator().manual_seed(5)
+    mk = lambda rows: torch.randn(B, rows, H, D, generator=g).to(torch.bfloat16).to(DEV)
+    t = sa.build_tree_topology(N, True, device=DEV)
+    q, qp, kp, vp = mk(N), mk(N - 1), mk(N - 1), mk(N - 1)
+    kfull = torch.zeros(B, 2 * N - 1, H, D, dtype=torch.bfloat16, device=DEV)
+    vfull = torch.zeros_like(kfull)
+    out = torch.zeros(B, N, H, D, dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        sa.build_tree(qp, kp, vp, kfull[:, :N], vfull[:, :N], out=kfull[:, N:], out2=vfull[:, N:])
+        fn.attention_forward(q, kfull, vfull, t["forward_idx"], t["forward_mask"], R, out=out)
+
+    kfull[:, :N], vfull[:, :N] = mk(N), mk(N)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                   # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(4):
+        for buf, rows in ((q, N), (qp, N - 1), (kp, N - 1), (vp, N - 1)):
+            buf.copy_(mk(rows))
+        kfull[:, :N].copy_(mk(N))
+        vfull[:, :N].copy_(mk(N))
+        graph.replay()
+        torch.cuda.synchronize()
+        got, nodes = out.clone(), kfull[:, N:].clone()
+        out.zero_()
+        kfull[:, N:].zero_()
+        step()                                   # eager, same inputs
+        torch.cuda.synchronize()
+        assert torch.equal(got, out) and torch.equal(nodes, kfull[:, N:]), "replay %d differs" % rep
+
+
+def test_lm_forward_replays_from_a_hip_graph():
+    """The whole decoder forward (projections by torch, tree and attention by the HIP kernels,
+    fused upper levels included) captured into one graph; replays on new token ids, with eager
+    forwards and synchronisations in between, equal the eager logits bit for bit."""
+    torch.manual_seed(0)
+    V, N, B = 211, 256, 2
+    model = sa.TransformerLM(V, 256, 4, 512, 2, dropout=0.0, window_size=8, activation="gelu", max_len=N)
+    model = model.to(DEV).to(torch.bfloat16).eval()
+    tok = torch.randint(0, V, (B, N), device=DEV)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                model(tok)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(tok)
+        for rep in range(3):
+            tok.copy_(torch.randint(0, V, (B, N), device=DEV))
+            graph.replay()
+            torch.cuda.synchronize()
+            got = out.clone()
+            want = model(tok)
+            torch.cuda.synchronize()
+            assert torch.equal(got, want), "replay %d differs" % rep
