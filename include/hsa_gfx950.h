@@ -65,7 +65,9 @@ const char *hsa_last_error(void);
  *   R           window radius: keys n-R..n+R (the reference's `window_size`)
  *   causal      used only when idx == NULL
  *   dtype       HSA_F32 / HSA_F16 / HSA_BF16
- *   algo        HSA_ATTN_*
+ *   algo        HSA_ATTN_*.  The MFMA tile kernels take canonical tables (idx == NULL), no
+ *               weights, R <= 32, 16 <= N <= 2^22, and head sizes 32 / 64 / 128 for the
+ *               16-bit types, 32 / 64 for fp32; everything else runs on the gather kernel
  */
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
@@ -76,8 +78,8 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
  * `stop_event` (hipEvent_t, created by the caller with timing enabled) are attached to the
  * span-attention dispatch and carry the kernel's begin and end timestamps, so
  * hipEventElapsedTime(start, stop) is the kernel duration without the idle gap between
- * consecutive launches that events recorded around a call include.  (The gather kernels record
- * the events around the launch instead.)  The reference times its kernels with torch events
+ * consecutive launches that events recorded around a call include.  (The gather kernels and the
+ * fp32 tile kernel record the events around the launch instead.)  The reference times its kernels with torch events
  * around the Python call (hierarchical_attention_project/Hierarchical_Attention_Triton_Test.py
  * :523-568); this is the same measurement taken at the dispatch.
  */
@@ -216,8 +218,10 @@ int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, cons
  *   q, dout, dq  [B, N, H, D];  k, v, dk, dv  [B, M, H, D], M >= 2N-1
  *   workspace    device memory of at least hsa_attn_bwd_workspace_bytes(...) bytes, provided by
  *                the caller (scratch only: nothing in it has to survive the call)
- *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit, head_dim 64, R <= 32:
- *                fp32 atomics for tree levels >= 4), else the deterministic gather kernels
+ *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit, head size 64 or 128,
+ *                R <= 32: a query-stationary pass, a key-stationary pass and a reduction of
+ *                per-block fp32 partial rows for tree levels >= 4), else the gather kernels;
+ *                both are deterministic (no atomics)
  */
 #include <stddef.h>
 size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo);

@@ -11,6 +11,15 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
                         bool want_weights);
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st);
+bool attn_tile_f32_eligible(int N, int M, int D, int L, int R, bool canonical, bool want_weights);
+int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *out, int B, int N, int M, int H,
+                           int D, int L, int R, int causal, hipStream_t st);
+
+// the MFMA tile kernels: 16-bit element types, or fp32 on the fp32 matrix instructions
+static bool tile_ok_for(int N, int M, int H, int D, int L, int R, int dtype, bool canonical, bool want_weights) {
+    if (dtype == HSA_F32) return attn_tile_f32_eligible(N, M, D, L, R, canonical, want_weights);
+    return attn_tile_eligible(N, M, H, D, L, R, dtype, canonical, want_weights);
+}
 
 }  // namespace hsa
 
@@ -18,7 +27,7 @@ extern "C" {
 
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype, int canonical_tables,
                            int want_weights) {
-    return hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, canonical_tables != 0, want_weights != 0) ? 1 : 0;
+    return hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical_tables != 0, want_weights != 0) ? 1 : 0;
 }
 
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
@@ -38,13 +47,22 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
         causal = (mask != nullptr);
     }
     hipStream_t st = (hipStream_t)stream;
-    const bool tile_ok = hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
+    const bool tile_ok = hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
     if (algo == HSA_ATTN_TILE && !tile_ok)
         return hsa::fail(HSA_ERR_UNSUPPORTED,
                          "tile kernel not available for N=%d H=%d D=%d L=%d R=%d dtype=%d canonical=%d",
                          N, H, D, L, R, dtype, (int)canonical);
-    if (tile_ok && algo != HSA_ATTN_GATHER)
+    if (tile_ok && algo != HSA_ATTN_GATHER) {
+        if (dtype == HSA_F32) {
+            // dispatch events are attached by the 16-bit launcher only: record around this one
+            const hsa::LaunchEvents ev = hsa::take_launch_events();
+            if (ev.start && ev.stop) (void)hipEventRecord(ev.start, st);
+            const int rc = hsa::attn_tile_f32_dispatch(q, k, v, out, B, N, M, H, D, L, R, causal ? 1 : 0, st);
+            if (ev.start && ev.stop) (void)hipEventRecord(ev.stop, st);
+            return rc;
+        }
         return hsa::attn_tile_dispatch(q, k, v, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0, dtype, st);
+    }
     // the gather kernels take no dispatch events: record around the call instead
     const hsa::LaunchEvents ev = hsa::take_launch_events();
     if (ev.start && ev.stop) (void)hipEventRecord(ev.start, st);

@@ -475,10 +475,36 @@ def test_attention_random_shapes(seed):
     assert_close(out, want, dtype, "B%d N%d H%d D%d R%d causal=%s %s" % (B, N, H, D, R, causal, dtype))
 
 
+F32_TILE_CASES = [(1, 16, 2, 64, 3), (2, 64, 3, 64, 16), (1, 256, 4, 32, 8), (2, 128, 2, 64, 20), (1, 512, 5, 32, 32),
+                  (1, 64, 2, 64, 0), (2, 1024, 8, 64, 16)]
+
+
+@pytest.mark.parametrize("case", F32_TILE_CASES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("strip", [None, "1", "2", "4"])
+def test_attention_tile_fp32_vs_oracle(case, causal, strip, monkeypatch):
+    """fp32 tensors on the fp32 matrix instructions: the 1e-5 bar against the fp64 oracle."""
+    B, N, H, D, R = case
+    if strip is not None:
+        monkeypatch.setenv("HSA_ATTN_TILE_SB", strip)
+    q, k, v = make_qkv(B, N, H, D, torch.float32, seed=N + R + D)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    o = oracle.topology_tables(N, causal)
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                               t["forward_mask"] if causal else None, R, algo="tile")
+    want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
+                                compute_dtype=torch.float64)
+    assert_close(out, want, torch.float32, "fp32 tile")
+    gath = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                                t["forward_mask"] if causal else None, R, algo="gather")
+    assert (out - gath).abs().max() < 2e-5
+
+
 def test_tile_is_the_default_for_the_headline_shape():
     from sparseattention_amd import _lib
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 1, 0) == 1
-    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_F32, 1, 0) == 0
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_F32, 1, 0) == 1
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 128, 11, 16, _lib.HSA_F32, 1, 0) == 0
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 0, 0) == 0
 
 
