@@ -30,7 +30,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int TQ = 16;            // queries per block
-constexpr int F32_WPB = 4;        // wavefronts per workgroup: one per SIMD, up to 512 VGPRs
+// wavefronts per workgroup: two per SIMD (256 registers each) where the variant fits, so that one
+// wavefront's matrix work overlaps the other's loads; else one per SIMD (up to 512 registers)
+template <int D, int NBW, bool CAUSAL> constexpr bool f32_fits_two_per_simd() { return D <= 32 || (CAUSAL && NBW <= 1); }
 constexpr int F32_MAX_LEVELS = 22;
 constexpr int F32_MAX_NBW = 2;
 constexpr float NEG_INF_F = -__builtin_inff();
@@ -43,7 +45,7 @@ struct TileF32Params {
     float scale_log2e;
 };
 
-template <int D, int NBW, bool CAUSAL, int SB>
+template <int D, int NBW, bool CAUSAL, int SB, int F32_WPB>
 __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Params p) {
     constexpr int DS = D / 4;                           // contraction steps of QK^T
     constexpr int NJ = D / 16;                          // 16-channel output tiles
@@ -54,7 +56,7 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
     constexpr int NLD = TQ / RPI;                       // load instructions per 16-row block
     constexpr int PITCH = D * 4 + 16;                   // LDS row pitch in bytes
     constexpr int BLK_BYTES = TQ * PITCH;
-    constexpr int WAVE_LDS = 5 * BLK_BYTES;             // q, k, v, near-tree k, near-tree v
+    constexpr int WAVE_LDS = 3 * BLK_BYTES;             // three operand blocks at a time
     __shared__ __align__(16) unsigned char smem[F32_WPB * WAVE_LDS];
 
     const int lane = threadIdx.x & 63;
@@ -224,26 +226,28 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
         const int row0 = leaf_row0(blk0 - NBW + c);
         load_block(Kb, row0, rk);
         load_block(Vb, row0, rv);
-        lds_put(2, rk);
-        lds_put(3, rv);
-        get_rows(2, Kl[c]);
-        get_cols(3, Vl[c]);
+        lds_put(0, rk);
+        lds_put(1, rv);
+        get_rows(0, Kl[c]);
+        get_cols(1, Vl[c]);
     }
 
     auto process = [&](Stage &sg, int blk, Stage &nsg, int next_blk) {
         const int q0 = blk * TQ;
         float Qf[DS], Kt[DS], Vt[NJ][4];
+        // three LDS blocks, reused: a wavefront's LDS operations execute in order, so a block may
+        // be overwritten as soon as the reads of its previous content have been issued
         lds_put(0, sg.q);
         lds_put(1, sg.k);
         lds_put(2, sg.v);
-        lds_put(3, sg.kt);
-        lds_put(4, sg.vt);
-        if (next_blk >= 0) request(nsg, next_blk);  // this block's raw registers are consumed
         get_rows(0, Qf);
         get_rows(1, Kl[NEWC]);
         get_cols(2, Vl[NEWC]);
-        get_rows(3, Kt);
-        get_cols(4, Vt);
+        lds_put(0, sg.kt);
+        lds_put(1, sg.vt);
+        if (next_blk >= 0) request(nsg, next_blk);  // this block's raw registers are consumed
+        get_rows(0, Kt);
+        get_cols(1, Vt);
 
         // scores, transposed: acc[i] = <key 4g+i of the block, query r16>
         f32x4 accL[NKL], accT = {0.f, 0.f, 0.f, 0.f}, accU = {0.f, 0.f, 0.f, 0.f};
@@ -337,16 +341,25 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
     }
 }
 
-template <int D, int NBW, bool CAUSAL>
-int launch_sb(const TileF32Params &p, int sb, hipStream_t st) {
-    const int nwg = (p.n_units + F32_WPB - 1) / F32_WPB;
+template <int D, int NBW, bool CAUSAL, int WPB>
+int launch_wpb(const TileF32Params &p, int sb, hipStream_t st) {
+    const int nwg = (p.n_units + WPB - 1) / WPB;
     switch (sb) {
-        case 1: attn_tile_f32_kernel<D, NBW, CAUSAL, 1><<<nwg, F32_WPB * 64, 0, st>>>(p); break;
-        case 2: attn_tile_f32_kernel<D, NBW, CAUSAL, 2><<<nwg, F32_WPB * 64, 0, st>>>(p); break;
-        case 4: attn_tile_f32_kernel<D, NBW, CAUSAL, 4><<<nwg, F32_WPB * 64, 0, st>>>(p); break;
+        case 1: attn_tile_f32_kernel<D, NBW, CAUSAL, 1, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
+        case 2: attn_tile_f32_kernel<D, NBW, CAUSAL, 2, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
+        case 4: attn_tile_f32_kernel<D, NBW, CAUSAL, 4, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
         default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
     }
     return check_launch("attn_tile_f32_kernel");
+}
+
+template <int D, int NBW, bool CAUSAL>
+int launch_sb(const TileF32Params &p, int sb, hipStream_t st) {
+    // eight wavefronts per workgroup only if that still gives every CU a workgroup
+    if constexpr (f32_fits_two_per_simd<D, NBW, CAUSAL>()) {
+        if (p.n_units >= 8 * 256) return launch_wpb<D, NBW, CAUSAL, 8>(p, sb, st);
+    }
+    return launch_wpb<D, NBW, CAUSAL, 4>(p, sb, st);
 }
 
 template <int D>
@@ -383,7 +396,7 @@ int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *ou
     const int NB = N / TQ;
     const int nbw = (R + TQ - 1) / TQ;
     const long block_units = (long)B * H * NB;
-    int sb = block_units >= 4 * 1024 ? 4 : (block_units >= 2 * 1024 ? 2 : 1);
+    int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
     if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
     if (!causal && nbw >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
     while (sb > NB) sb >>= 1;
