@@ -1,0 +1,4 @@
+#include "hsa_attn_bwd_tile_inst.h"
+namespace hsa {
+HSA_BWD_TILE_INSTANTIATE(F16, 32)
+}  // namespace hsa

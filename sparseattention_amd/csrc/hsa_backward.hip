@@ -623,7 +623,7 @@ __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, ty
 // ---------------------------------------------------------------- tile backward dispatch
 static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype) {
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
-    if (D != 64 && D != 128) return false;
+    if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
     if ((R + TILE_Q - 1) / TILE_Q > 2) return false;
     return true;
@@ -652,8 +652,10 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.n_units = (int)units;
     p.scale = 1.0f / sqrtf((float)D);
     p.scale_log2e = 1.4426950408889634f * p.scale;
-    int rc = D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, (R + TILE_Q - 1) / TILE_Q, causal != 0, st)
-                     : attn_bwd_tile_launch_td<T, 128>(p, (R + TILE_Q - 1) / TILE_Q, causal != 0, st);
+    const int nbw = (R + TILE_Q - 1) / TILE_Q;
+    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, st)
+           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, st)
+                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, st);
     if (rc != HSA_OK) return rc;
     const int first = level_offset(N, 4);
     const size_t n_fin = (size_t)B * (M - first) * H * D;
