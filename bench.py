@@ -35,6 +35,9 @@ def parse():
     ap.add_argument("--workload", default="cfg3", choices=sorted(WORKLOADS) + ["cfg4"])
     ap.add_argument("--noncausal", action="store_true")
     ap.add_argument("--seq-len", type=int, default=0, help="override the workload's N (a power of two)")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="a step is the span attention alone, on span nodes drawn i.i.d. like the leaves "
+                         "(isolates the attention kernel; the tree build is not run)")
     ap.add_argument("--sets", type=int, default=0, help="buffer sets to rotate through (0 = enough to exceed 512 MB)")
     ap.add_argument("--streams", type=int, default=2,
                     help="HIP streams the steps alternate between (each step is an independent batch)")
@@ -283,8 +286,15 @@ def main():
 
     kev = [(new_event(), new_event()) for _ in range(args.steps)]
 
+    if args.attention_only:
+        for s_ in sets:
+            s_["kfull"][:, N:] = (torch.randn(B, N - 1, H, D, generator=g) * scale).to(torch.bfloat16).to(dev)
+            s_["vfull"][:, N:] = (torch.randn(B, N - 1, H, D, generator=g) * scale).to(torch.bfloat16).to(dev)
+        torch.cuda.synchronize()
+    tree_fwd = (lambda *a: 0) if args.attention_only else lib.hsa_build_tree_fwd
+
     def step(i, ev=None):
-        rc = lib.hsa_build_tree_fwd(*targs[i % nsets])
+        rc = tree_fwd(*targs[i % nsets])
         if ev is None:
             rc |= lib.hsa_attn_fwd(*aargs[i % nsets])
         else:
@@ -292,7 +302,7 @@ def main():
         return rc
 
     def step_p(i):
-        rc = lib.hsa_build_tree_fwd(*targs_p[i % nsets])
+        rc = tree_fwd(*targs_p[i % nsets])
         rc |= lib.hsa_attn_fwd(*aargs_p[i % nsets])
         return rc
 
@@ -364,7 +374,7 @@ def main():
     torch.cuda.synchronize()
     for i in range(K):
         a = i % nsets
-        lib.hsa_build_tree_fwd(*targs[a])
+        tree_fwd(*targs[a])
         ev[i][0].record(stream)
         lib.hsa_attn_fwd(*aargs[a])
         ev[i][1].record(stream)
@@ -424,7 +434,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, H, N, D, R, causal, scale, args.cpu_seconds)
-    if args.workload != "cfg3" or not causal or args.seq_len:
+    if args.attention_only:
+        result["config"]["workload"] = result["config"]["workload"].replace(
+            "step = tree build + span attention forward", "step = span attention forward alone (i.i.d. span nodes)")
+    if args.workload != "cfg3" or not causal or args.seq_len or args.attention_only:
         result["metric"] = "attn fwd queries/sec + % HBM roofline, " + desc
     print(json.dumps(result))
 
