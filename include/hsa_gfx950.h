@@ -230,6 +230,24 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
                  int L, int R, int causal, int dtype, int algo, void *stream);
 
 /*
+ * hsa_attn_bwd for callers that cannot allocate device memory or hand over a workspace (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference: its backward allocates its workspaces through torch
+ * (hierarchical_attention/ops/functional.py:171-264).  Same arguments, kernels and results as
+ * hsa_attn_bwd, but the scratch is a buffer of HSA_ATTN_BWD_STATIC_BYTES that is part of the
+ * library's device image (each GPU the library runs on holds one until the process ends); the
+ * call allocates nothing.  Problems with hsa_attn_bwd_workspace_bytes(...) above that size are
+ * refused with HSA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's buffer: calls that
+ * overlap on one GPU (two streams, two host threads) race; calls on one stream do not.
+ * Nothing in the buffer has to be cleared between calls.
+ */
+#define HSA_ATTN_BWD_STATIC_BYTES (32u << 20)
+size_t hsa_attn_bwd_static_capacity(void);
+int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                        void *dv, int B, int N, int M, int H, int D, int L, int R, int causal, int dtype,
+                        int algo, void *stream);
+
+/*
  * Backward of the initial span nodes (the reference differentiates generate_span_input_Y,
  * hierarchical_attention/ops/topology.py:153-169, through torch autograd):
  *   dx[b, n, :] = sum_{l=1..log2 N} 2^-l * dy[b, level l node n >> l, :]

@@ -60,6 +60,10 @@ def _declare(lib):
     lib.hsa_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.hsa_attn_bwd.argtypes = [P] * 8 + [ctypes.c_size_t] + [I] * 10 + [P]
     lib.hsa_attn_bwd.restype = I
+    lib.hsa_attn_bwd_static_capacity.argtypes = []
+    lib.hsa_attn_bwd_static_capacity.restype = ctypes.c_size_t
+    lib.hsa_attn_bwd_static.argtypes = [P] * 7 + [I] * 10 + [P]
+    lib.hsa_attn_bwd_static.restype = I
     lib.hsa_span_input_y_bwd.argtypes = [P, P, I, I, I, I, P]
     lib.hsa_span_input_y_bwd.restype = I
 

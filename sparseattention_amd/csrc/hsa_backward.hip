@@ -13,6 +13,8 @@
 //                     dK = sum dS Q, dV = sum P dO in fp32, written once in the element type.
 //                 Canonical complete-binary-tree tables only.
 //  span nodes     dx[n] = sum_l 2^-l dY[level l, n >> l].
+#include <mutex>
+
 #include "hsa_attn_bwd_tile.h"
 
 namespace hsa {
@@ -721,6 +723,56 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
         case HSA_BF16: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
     }
     return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+// ---- hsa_attn_bwd for callers that must not allocate ---------------------------------------------
+// The workspace of hsa_attn_bwd lives in this file-scope device array instead of caller memory.
+// Every device the library's code object is loaded on holds its own copy at its own address;
+// host code never uses the array's name as an address, only what hipGetSymbolAddress returned
+// for the device that is current.
+static __device__ __align__(256) unsigned char scratch[HSA_ATTN_BWD_STATIC_BYTES];
+
+namespace hsa {
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[kMaxDevices];  // per device, filled on the first call there
+
+static int scratch_for_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(HSA_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(HSA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return HSA_OK;
+}
+}  // namespace hsa
+
+size_t hsa_attn_bwd_static_capacity(void) { return (size_t)HSA_ATTN_BWD_STATIC_BYTES; }
+
+int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                        void *dv, int B, int N, int M, int H, int D, int L, int R, int causal, int dtype,
+                        int algo, void *stream) {
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
+    HSA_REQUIRE(L >= 0 && R >= 0, "bad L=%d R=%d", L, R);
+    const size_t need = hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, dtype, algo);
+    if (need > (size_t)HSA_ATTN_BWD_STATIC_BYTES)
+        return hsa::fail(HSA_ERR_UNSUPPORTED,
+                         "problem needs %zu bytes of scratch, the built-in buffer holds %zu: use hsa_attn_bwd "
+                         "with a caller-provided workspace", need, (size_t)HSA_ATTN_BWD_STATIC_BYTES);
+    void *ws = nullptr;
+    const int rc = hsa::scratch_for_current_device(&ws);
+    if (rc != HSA_OK) return rc;
+    // the kernels write every workspace entry before they read it: nothing to clear between calls
+    return hsa_attn_bwd(q, k, v, dout, dq, dk, dv, ws, (size_t)HSA_ATTN_BWD_STATIC_BYTES, B, N, M, H, D, L, R,
+                        causal, dtype, algo, stream);
 }
 
 int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtype, void *stream) {
