@@ -88,6 +88,19 @@ int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_
                        int D, int L, int R, int causal, int dtype, int algo, void *stream,
                        void *start_event, void *stop_event);
 
+/*
+ * Launch parameters of the 16-bit MFMA tile kernel, for experiments (no counterpart in the
+ * reference, whose Triton launch fixes one program per query, ops/functional.py:143-161).
+ *   strip_blocks     16-query blocks one wavefront walks: 1, 2 or 4; 0 = chosen by problem size
+ *   waves_per_group  wavefronts per workgroup, 1..8
+ *   xcd_remap        0 = workgroup ids map to strips in order, 1 = neighbouring strips share an XCD
+ *   alternate        0 = every strip walks upwards, 1 = neighbouring strips walk towards each other
+ * An argument of -1 keeps the current value.  Process-wide; the initial values come from the
+ * environment variables HSA_ATTN_TILE_SB / _WPB / _SWZ / _ALT, read once.  Results do not depend
+ * on any of them.
+ */
+int hsa_attn_tile_tune(int strip_blocks, int waves_per_group, int xcd_remap, int alternate);
+
 /* 1 if HSA_ATTN_AUTO would pick the MFMA tile kernel for this problem, else 0. */
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype,
                            int canonical_tables, int want_weights);

@@ -19,8 +19,17 @@ tests/test_oracle.py):
                          special cases (Q=0, constant V, N=2, causal row 0)  PINNED
   build_parent_nodes_ref F.softmax closed form, Q=0 mean, C brute force   PINNED
   span_input_y_ref       block-mean closed form                           PINNED
-  cross_update_y_ref /   composition of the above with torch.nn.functional.linear,
-  update_x_from_y_ref    identity-projection reductions to the op oracles PINNED
+  cross_update_y_ref /   scalar per-parent / per-query loops written from the module's
+  update_x_from_y_ref    definition with random, distinct weights and biases; the
+                         uniform-softmax closed forms (Wq = 0: a linear recursion in
+                         Wv, leaves reach level l through Wv^l / 3^l); identity-
+                         projection reductions to the op oracles
+                         (tests/test_oracle_modules.py)                   PINNED
+  lm_forward_ref         (oracle/lm_ref.py) no layers = tied read-out of the scaled,
+                         position-encoded embedding; silent attention = pre-norm FFN
+                         stack; one layer wired by hand from the pinned module
+                         oracles, told apart from four mis-wirings; causality
+                         (tests/test_oracle_modules.py)                   PINNED
 """
 from __future__ import annotations
 

@@ -11,6 +11,7 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
                         bool want_weights);
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st);
+int attn_tile_tune(int sb, int wpb, int swizzle, int alternate);
 bool attn_tile_f32_eligible(int N, int M, int D, int L, int R, bool canonical, bool want_weights);
 int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *out, int B, int N, int M, int H,
                            int D, int L, int R, int causal, hipStream_t st);
@@ -24,6 +25,10 @@ static bool tile_ok_for(int N, int M, int H, int D, int L, int R, int dtype, boo
 }  // namespace hsa
 
 extern "C" {
+
+int hsa_attn_tile_tune(int strip_blocks, int waves_per_group, int xcd_remap, int alternate) {
+    return hsa::attn_tile_tune(strip_blocks, waves_per_group, xcd_remap, alternate);
+}
 
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype, int canonical_tables,
                            int want_weights) {
@@ -47,7 +52,11 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
         causal = (mask != nullptr);
     }
     hipStream_t st = (hipStream_t)stream;
-    const bool tile_ok = hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
+    bool tile_ok = hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
+    // the tile kernels move 16-byte pieces: tensors at other addresses (a view at an odd element
+    // offset) go to the gather kernel unless the tile kernel was asked for by name
+    const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0;
+    if (!aligned && algo != HSA_ATTN_TILE) tile_ok = false;
     if (algo == HSA_ATTN_TILE && !tile_ok)
         return hsa::fail(HSA_ERR_UNSUPPORTED,
                          "tile kernel not available for N=%d H=%d D=%d L=%d R=%d dtype=%d canonical=%d",

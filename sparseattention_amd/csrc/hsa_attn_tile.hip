@@ -3,9 +3,46 @@
 
 #include <stdlib.h>
 
+#include <atomic>
+
 namespace hsa {
 
 constexpr int TILE_MAX_NBW = 2;
+
+// Experiment knobs of the tile launch: strip length in query blocks (0 = by problem size),
+// wavefronts per workgroup, XCD remap on/off, alternating strip direction on/off.  Initialised
+// once per process from HSA_ATTN_TILE_SB / _WPB / _SWZ / _ALT, changed afterwards only through
+// hsa_attn_tile_tune; a launch reads four atomics, never the environment.
+struct TileKnobs {
+    std::atomic<int> sb{0}, wpb{8}, swizzle{1}, alternate{1};
+    TileKnobs() {
+        if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+        if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) swizzle = atoi(e) != 0;
+        if (const char *e = getenv("HSA_ATTN_TILE_ALT")) alternate = atoi(e) != 0;
+        if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
+    }
+};
+static TileKnobs &tile_knobs() {
+    static TileKnobs k;
+    return k;
+}
+
+// the two knobs the fp32 tile launch shares
+void attn_tile_knobs_sb_swizzle(int *sb, int *swizzle) {
+    *sb = tile_knobs().sb;
+    *swizzle = tile_knobs().swizzle;
+}
+
+int attn_tile_tune(int sb, int wpb, int swizzle, int alternate) {
+    if (!(sb == -1 || sb == 0 || sb == 1 || sb == 2 || sb == 4)) return fail(HSA_ERR_INVALID, "strip length %d", sb);
+    if (!(wpb == -1 || (wpb >= 1 && wpb <= 8))) return fail(HSA_ERR_INVALID, "wavefronts per workgroup %d", wpb);
+    TileKnobs &k = tile_knobs();
+    if (sb >= 0) k.sb = sb;
+    if (wpb >= 0) k.wpb = wpb;
+    if (swizzle >= 0) k.swizzle = swizzle != 0;
+    if (alternate >= 0) k.alternate = alternate != 0;
+    return HSA_OK;
+}
 
 bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
                         bool want_weights) {
@@ -29,24 +66,22 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     p.out = (uint16_t *)out;
     p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
     const int NB = N / TILE_Q;
+    TileKnobs &knobs = tile_knobs();
     // strip length: long enough to amortise the halo and to prefetch, short enough to give
     // every SIMD of the 256 CUs at least two wavefronts
     const long block_units = (long)B * H * NB;
     int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
-    if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+    if (const int forced = knobs.sb) sb = forced;
     if (!causal && (R + TILE_Q - 1) / TILE_Q >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
     while (sb > NB) sb >>= 1;  // NB is a power of two
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;
     if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.n_units = (int)units;
-    p.xcd_swizzle = 1;
-    if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) p.xcd_swizzle = atoi(e);
-    p.alternate = 1;
-    if (const char *e = getenv("HSA_ATTN_TILE_ALT")) p.alternate = atoi(e);
+    p.xcd_swizzle = knobs.swizzle;
+    p.alternate = knobs.alternate;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
-    int wpb = 8;
-    if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
+    const int wpb = knobs.wpb;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (dtype == HSA_BF16) {
         if (D == 32) return attn_tile_launch_td<BF16, 32>(p, nbw, causal != 0, sb, wpb, st);

@@ -377,6 +377,8 @@ int launch_d(const TileF32Params &p, int nbw, bool causal, int sb, hipStream_t s
 
 }  // namespace
 
+void attn_tile_knobs_sb_swizzle(int *sb, int *swizzle);  // hsa_attn_tile.hip
+
 bool attn_tile_f32_eligible(int N, int M, int D, int L, int R, bool canonical, bool want_weights) {
     if (!canonical || want_weights) return false;
     if (D != 32 && D != 64) return false;
@@ -397,15 +399,16 @@ int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *ou
     const int nbw = (R + TQ - 1) / TQ;
     const long block_units = (long)B * H * NB;
     int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
-    if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+    int forced_sb = 0, swizzle = 1;
+    attn_tile_knobs_sb_swizzle(&forced_sb, &swizzle);
+    if (forced_sb) sb = forced_sb;
     if (!causal && nbw >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
     while (sb > NB) sb >>= 1;
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;
     if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.n_units = (int)units;
-    p.xcd_swizzle = 1;
-    if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) p.xcd_swizzle = atoi(e);
+    p.xcd_swizzle = swizzle;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
     if (D == 32) return launch_d<32>(p, nbw, causal != 0, sb, st);
     return launch_d<64>(p, nbw, causal != 0, sb, st);

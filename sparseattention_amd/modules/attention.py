@@ -73,17 +73,50 @@ class HierarchicalAttention(nn.Module):
     def _heads(self, t: torch.Tensor) -> torch.Tensor:
         return t.view(t.shape[0], -1, self.num_heads, self.head_dim)
 
-    def _fused_weight(self, name: str, layers, packed: bool = False) -> torch.Tensor:
-        """Weights of several bias-free projections stacked along the output dimension, so one
-        GEMM computes them all (packed: key / value weights in the operand order of the fused
-        upper levels); rebuilt when any of them has been written to or moved."""
-        key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype) for m in layers)
+    def reset_fused_weights(self):
+        """Drops the cached stacked / packed projection weights of the no-autograd path.  The cache
+        notices optimizer steps, `load_state_dict`, `.to()` and `train()` by itself; call this after
+        writing to a weight through `.data` (such writes leave no trace on the tensor)."""
+        self._fused.clear()
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._fused.clear()
+        return super()._load_from_state_dict(*args, **kwargs)
+
+    def _apply(self, fn, *args, **kwargs):
+        self._fused.clear()
+        return super()._apply(fn, *args, **kwargs)
+
+    def train(self, mode: bool = True):
+        self._fused.clear()
+        return super().train(mode)
+
+    def _fused_weight(self, name: str, layers, dtype: torch.dtype, packed: bool = False) -> torch.Tensor:
+        """Weights of several bias-free projections, cast to `dtype` and stacked along the output
+        dimension, so one GEMM computes them all (packed: key / value weights in the operand order
+        of the fused upper levels); rebuilt when any of them has been written to or moved."""
+        key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype) for m in layers) + (dtype,)
         hit = self._fused.get(name)
         if hit is None or hit[0] != key:
-            ws = [m.weight.detach() for m in layers]
+            ws = [m.weight.detach().to(dtype) for m in layers]
             hit = (key, pack_kv_weights(ws[0], ws[1], self.num_heads) if packed else torch.cat(ws, dim=0))
             self._fused[name] = hit
         return hit[1]
+
+    @staticmethod
+    def _compute_dtype(t: torch.Tensor) -> torch.dtype:
+        """Element type the projections produce: the autocast type inside `torch.autocast` (the
+        reference's evaluation loop runs under it with fp32 activations and weights), else the
+        activations' own type."""
+        if t.is_cuda and torch.is_autocast_enabled("cuda"):
+            return torch.get_autocast_dtype("cuda")
+        return t.dtype
+
+    def _needs_autograd(self, tensors, layers) -> bool:
+        if not torch.is_grad_enabled():
+            return False
+        return any(t.requires_grad for t in tensors) or any(
+            p.requires_grad for m in layers for p in m.parameters())
 
     def _cross_update_Y_direct(self, x: torch.Tensor, y_in: torch.Tensor) -> torch.Tensor:
         """cross_update_Y without autograd and without dropout: the three projections of the span
@@ -95,11 +128,14 @@ class HierarchicalAttention(nn.Module):
         B, N, D = x.shape
         H, Dh = self.num_heads, self.head_dim
         _lib.require_gpu(x, y_in)
-        x, y_in = x.contiguous(), y_in.contiguous()
-        qkv = F.linear(y_in, self._fused_weight("qkv_y", (self.Wq_y, self.Wk_y, self.Wv_y)))  # [B, N-1, 3D]
-        w_kv = self._fused_weight("kv_y", (self.Wk_y, self.Wv_y))
-        y_new = torch.empty((B, N - 1, D), dtype=x.dtype, device=x.device)
-        blocks = torch.empty(B * (N - 1) * D, dtype=x.dtype, device=x.device)  # level-major
+        cdt = self._compute_dtype(x)
+        x, y_in = x.to(cdt).contiguous(), y_in.to(cdt).contiguous()
+        qkv = F.linear(y_in, self._fused_weight("qkv_y", (self.Wq_y, self.Wk_y, self.Wv_y), cdt))  # [B, N-1, 3D]
+        w_kv = self._fused_weight("kv_y", (self.Wk_y, self.Wv_y), cdt)
+        # every buffer the kernels address by raw pointer has the one element type
+        assert qkv.dtype == cdt and qkv.is_contiguous(), "projection result has an unexpected layout"
+        y_new = torch.empty((B, N - 1, D), dtype=cdt, device=x.device)
+        blocks = torch.empty(B * (N - 1) * D, dtype=cdt, device=x.device)  # level-major
         # the level loop works on raw addresses: the operands are fixed column slices of qkv and
         # of each level's k/v projection, so no tensor views are made per level
         es = x.element_size()
@@ -114,13 +150,15 @@ class HierarchicalAttention(nn.Module):
             for P in self.sizes:
                 if 2 * P <= top_rows:
                     # the remaining levels fit one workgroup per batch: a single launch
-                    w_top = self._fused_weight("kv_y_packed", (self.Wk_y, self.Wv_y), packed=True)
+                    w_top = self._fused_weight("kv_y_packed", (self.Wk_y, self.Wv_y), cdt, packed=True)
+                    assert src.dtype == cdt and src.is_contiguous() and w_top.dtype == cdt
                     rc = _lib.lib().hsa_cross_update_top_fwd(
                         src.data_ptr(), qkv_p + off * 3 * D * es, w_top.data_ptr(), out_p + off * D * es,
                         B, 2 * P, H, Dh, 0, (N - 1) * 3 * D, 3 * D, (N - 1) * D, D, code, stream)
                     _lib.check(rc, "hsa_cross_update_top_fwd")
                     break
                 kv = F.linear(src, w_kv)  # [B, 2P, 2D]
+                assert kv.dtype == cdt and kv.is_contiguous(), "projection result has an unexpected layout"
                 par, kv_p, lvl_p = qkv_p + off * 3 * D * es, kv.data_ptr(), blk_p + B * off * D * es
                 rc = fwd(par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es, lvl_p,
                          out_p + off * D * es, B, P, H, Dh,
@@ -140,8 +178,7 @@ class HierarchicalAttention(nn.Module):
         if self.sizes is None or self.sizes[0] != N // 2:
             self.sizes, self.offsets = self._build_level_info(N)
 
-        grad = torch.is_grad_enabled() and (x.requires_grad or y_in.requires_grad
-                                            or self.Wq_y.weight.requires_grad)
+        grad = self._needs_autograd((x, y_in), (self.Wq_y, self.Wk_y, self.Wv_y))
         if not grad and not (self.training and self.dropout.p > 0):
             return self._cross_update_Y_direct(x, y_in)
 
@@ -164,17 +201,21 @@ class HierarchicalAttention(nn.Module):
         B, N, D = x.shape
         assert y is not None, "y (parents) cannot be None during top-down update"
         q = self._heads(self.Wq_x(x))
-        grad = torch.is_grad_enabled() and (x.requires_grad or y.requires_grad
-                                            or self.Wk_x.weight.requires_grad)
+        grad = self._needs_autograd((x, y), (self.Wq_x, self.Wk_x, self.Wv_x))
         if not grad and not (self.training and self.dropout.p > 0) and y.size(1) == N - 1:
             # leaves and span nodes are projected straight into their rows of the [B, 2N-1, D]
-            # key / value buffers (batched GEMMs with a strided output): no concatenated input
-            k = torch.empty((B, 2 * N - 1, D), dtype=x.dtype, device=x.device)
+            # key / value buffers (batched GEMMs with a strided output): no concatenated input.
+            # Everything is brought to the type of q first (under autocast the activations and
+            # weights are fp32 while the projections come out in the autocast type; GEMMs with an
+            # `out=` are not autocast)
+            cdt = q.dtype
+            xc, yc = x.to(cdt), y.to(cdt)
+            k = torch.empty((B, 2 * N - 1, D), dtype=cdt, device=x.device)
             v = torch.empty_like(k)
             for lin, dst in ((self.Wk_x, k), (self.Wv_x, v)):
-                wt = lin.weight.t().unsqueeze(0).expand(B, D, D)
-                torch.bmm(x, wt, out=dst[:, :N])
-                torch.bmm(y, wt, out=dst[:, N:])
+                wt = lin.weight.detach().to(cdt).t().unsqueeze(0).expand(B, D, D)
+                torch.bmm(xc, wt, out=dst[:, :N])
+                torch.bmm(yc, wt, out=dst[:, N:])
             k, v = self._heads(k), self._heads(v)
         else:
             xy = torch.cat([x, y], dim=1)

@@ -35,10 +35,18 @@ def verify_tables(idx_table: torch.Tensor, mask_table: Optional[torch.Tensor]) -
     N, L = idx_table.shape
     if N < 1 or (N & (N - 1)) != 0 or L != N.bit_length() - 1:
         return False
+    if _topo.known_other(idx_table) or _topo.known_other(mask_table):
+        return False
+    if torch.cuda.is_current_stream_capturing():
+        return False  # the comparison synchronises: under graph capture unknown tables stay unknown
     canon = _topo.build_tree_topology(N, mask_table is not None, idx_table.device)
     ok = bool(torch.equal(idx_table.to(torch.int32), canon["forward_idx"]))
-    if ok and mask_table is not None:
+    if not ok:
+        _topo.remember_other(idx_table)
+    elif mask_table is not None:
         ok = bool(torch.equal(mask_table.to(torch.bool), canon["forward_mask"]))
+        if not ok:
+            _topo.remember_other(mask_table)
     if ok and idx_table.dtype == torch.int32:
         _topo._remember(idx_table, "idx", N, mask_table is not None)
         if mask_table is not None and mask_table.dtype == torch.bool:

@@ -25,6 +25,24 @@ def _remember(t: torch.Tensor, kind: str, n: int, causal: bool):
     _KNOWN[key] = (weakref.ref(t, lambda _r, k=key: _KNOWN.pop(k, None)), t._version, kind, n, causal)
 
 
+# Tables of unknown origin that were compared with the canonical ones and differ:
+# id(tensor) -> (weakref, version).  Saves the comparison (a host sync) on later calls.
+_KNOWN_OTHER: Dict[int, tuple] = {}
+
+
+def remember_other(t: torch.Tensor):
+    key = id(t)
+    _KNOWN_OTHER[key] = (weakref.ref(t, lambda _r, k=key: _KNOWN_OTHER.pop(k, None)), t._version)
+
+
+def known_other(t: Optional[torch.Tensor]) -> bool:
+    """True if `t` was found to differ from the canonical table and has not been written since."""
+    if t is None:
+        return False
+    rec = _KNOWN_OTHER.get(id(t))
+    return rec is not None and rec[0]() is t and rec[1] == t._version
+
+
 def known_table(t: Optional[torch.Tensor], kind: str):
     """(N, causal) if `t` is an unmodified canonical table of that kind, else None."""
     if t is None:
