@@ -176,7 +176,8 @@ int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv,
  * Out_l = build_parent_nodes(Qp_l, Kp_l, Vp_l, Out_{l-1}, Out_{l-1}) of the op at
  * hierarchical_attention/ops/functional.py:271-272, i.e. the level loop of
  * hierarchical_attention/modules/attention.py:119-157 with an identity map
- * between levels).  Intermediate levels stay on chip.
+ * between levels).  Intermediate levels stay on chip; one kernel launch for the whole tree
+ * (see hsa_build_tree_tune for the conditions).
  *
  *   qp, kp, vp  [B, N-1, H, D] level-concatenated (level 1 first, root last)
  *   k_leaf, v_leaf [B, N, H, D]
@@ -189,6 +190,24 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
                        const void *v_leaf, void *out, void *out2, int B, int N, int H, int D,
                        int64_t qp_bs, int64_t kp_bs, int64_t vp_bs, int64_t kleaf_bs,
                        int64_t vleaf_bs, int64_t out_bs, int64_t out2_bs, int dtype, void *stream);
+
+/*
+ * How hsa_build_tree_fwd runs, for experiments and tests (no counterpart in the reference).
+ *   mode               0 = always a few levels per launch;
+ *                      1 = (default) the whole tree in one kernel where that is faster: shapes
+ *                          whose workgroups all fit on the chip at once;
+ *                      2 = one kernel wherever the shape allows it (16-byte rows, power-of-two
+ *                          head count, N >= 8).
+ *                      In the single launch, workgroups finish their own subtrees and the last
+ *                      one of each group to arrive continues upwards, counted by arrival
+ *                      counters inside the library image (one slice per stream; a launch on a
+ *                      capturing stream, or on the 33rd distinct stream, takes the multi-launch
+ *                      path).
+ *   workgroup_threads  64 / 128 / 256 / 512: workgroup size of the single launch, 0 = by
+ *                      problem size (default)
+ * -1 keeps a value.  Process-wide.  Results do not depend on either.
+ */
+int hsa_build_tree_tune(int mode, int workgroup_threads);
 
 /*
  * Topology tables.  Replaces build_tree_topology

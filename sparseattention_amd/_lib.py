@@ -50,6 +50,8 @@ def _declare(lib):
     lib.hsa_cross_update_top_fwd.restype = I
     lib.hsa_build_tree_fwd.argtypes = [P] * 7 + [I] * 4 + [I64] * 7 + [I, P]
     lib.hsa_build_tree_fwd.restype = I
+    lib.hsa_build_tree_tune.argtypes = [I, I]
+    lib.hsa_build_tree_tune.restype = I
     lib.hsa_topology_host.argtypes = [I, I, P, P, P]
     lib.hsa_topology_host.restype = I
     lib.hsa_topology_device.argtypes = [I, I, P, P, P, P]

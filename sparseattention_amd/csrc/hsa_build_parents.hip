@@ -5,39 +5,9 @@
 // (one or more whole token rows) per load instruction.  The three dot products
 // are reduced inside the group with xor shuffles; the 3-way softmax and the
 // weighted sum of the value rows stay in fp32 registers.
-#include "hsa_common.h"
+#include "hsa_build_vec.h"
 
 namespace hsa {
-
-template <typename T, int VEC> struct Pack { typename T::storage e[VEC]; };
-
-template <typename T, int VEC>
-__device__ __forceinline__ void load_vec(const typename T::storage *p, float (&f)[VEC]) {
-    if constexpr (VEC == 1) {
-        f[0] = to_float<T>(p[0]);
-    } else {
-        using P = Pack<T, VEC>;
-        P v = *reinterpret_cast<const P *>(p);
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) f[i] = to_float<T>(v.e[i]);
-    }
-}
-
-template <typename T, int VEC>
-__device__ __forceinline__ void store_vec(typename T::storage *p, const float (&f)[VEC]) {
-    if constexpr (VEC == 1) {
-        p[0] = from_float<T>(f[0]);
-    } else {
-        using P = Pack<T, VEC>;
-        P v;
-#pragma unroll
-        for (int i = 0; i < VEC; ++i) v.e[i] = from_float<T>(f[i]);
-        static_assert(sizeof(P) == 16, "vector path moves 16 bytes per lane");
-        // regular store: the rows are read again by the next launch (a streaming store makes the
-        // tree build itself ~8% faster and the attention kernel after it as much slower)
-        *reinterpret_cast<P *>(p) = v;
-    }
-}
 
 // Batch and row strides (in elements) of the seven operands of one level, in the order
 // qp, kp, vp, kc, vc, out, out2.  A row stride wider than H*D reads a column slice of a
@@ -189,33 +159,45 @@ build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename 
     const size_t rs = (size_t)H * D;
     const size_t hd = (size_t)h * D + (dok ? d : 0);
 
-    // Every row this subtree needs is requested up front (children first, then the parent
-    // q/k/v rows of all TL levels): one memory round trip instead of one per level.
+    // Every row this subtree needs is requested up front, in the order the results are used
+    // (first level parent by parent: its two children and its own q/k/v; then the upper levels).
+    // Loads return in order, so the first parents are computed while later rows still arrive.
     using P = Pack<T, VEC>;
     P rck[NC], rcv[SHARED ? 1 : NC], rq[NC - 1], rk[NC - 1], rv[NC - 1];
     {
         const S *kc = Kc + (size_t)b * kc_bs + (size_t)sub * NC * rs + hd;
         const S *vc = Vc + (size_t)b * vc_bs + (size_t)sub * NC * rs + hd;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            rck[c] = *reinterpret_cast<const P *>(kc + (size_t)c * rs);
-            if (!SHARED) rcv[c] = *reinterpret_cast<const P *>(vc + (size_t)c * rs);
-        }
-    }
-#pragma unroll
-    for (int j = 1; j <= TL; ++j) {
-        const int np = NC >> j;
-        const int base = NC - 2 * np;  // slot of this level's first parent: 0, NC/2, 3NC/4, ...
-        const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + (size_t)sub * np;
+        const size_t lrow = (size_t)(level_offset(N, lvl0 + 1) - N) + (size_t)sub * (NC / 2);
         const S *q = Qp + (size_t)b * qp_bs + lrow * rs + hd;
         const S *kp = Kp + (size_t)b * kp_bs + lrow * rs + hd;
         const S *vp = Vp + (size_t)b * vp_bs + lrow * rs + hd;
 #pragma unroll
         for (int i = 0; i < NC / 2; ++i) {
+            rq[i] = load_once<P>(q + (size_t)i * rs);
+            rck[2 * i] = load_once<P>(kc + (size_t)(2 * i) * rs);
+            rck[2 * i + 1] = load_once<P>(kc + (size_t)(2 * i + 1) * rs);
+            rk[i] = load_once<P>(kp + (size_t)i * rs);
+            if (!SHARED) {
+                rcv[2 * i] = load_once<P>(vc + (size_t)(2 * i) * rs);
+                rcv[2 * i + 1] = load_once<P>(vc + (size_t)(2 * i + 1) * rs);
+            }
+            rv[i] = load_once<P>(vp + (size_t)i * rs);
+        }
+    }
+#pragma unroll
+    for (int j = 2; j <= TL; ++j) {
+        const int np = NC >> j;
+        const int base = NC - 2 * np;  // slot of this level's first parent: NC/2, 3NC/4, ...
+        const size_t lrow = (size_t)(level_offset(N, lvl0 + j) - N) + (size_t)sub * np;
+        const S *q = Qp + (size_t)b * qp_bs + lrow * rs + hd;
+        const S *kp = Kp + (size_t)b * kp_bs + lrow * rs + hd;
+        const S *vp = Vp + (size_t)b * vp_bs + lrow * rs + hd;
+#pragma unroll
+        for (int i = 0; i < NC / 4; ++i) {
             if (i < np) {
-                rq[base + i] = *reinterpret_cast<const P *>(q + (size_t)i * rs);
-                rk[base + i] = *reinterpret_cast<const P *>(kp + (size_t)i * rs);
-                rv[base + i] = *reinterpret_cast<const P *>(vp + (size_t)i * rs);
+                rq[base + i] = load_once<P>(q + (size_t)i * rs);
+                rk[base + i] = load_once<P>(kp + (size_t)i * rs);
+                rv[base + i] = load_once<P>(vp + (size_t)i * rs);
             }
         }
     }
@@ -223,15 +205,10 @@ build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename 
     // keep every request ahead of the first use
     __builtin_amdgcn_sched_barrier(0);
 
-    float ck[NC][VEC], cv[NC][VEC];
-#pragma unroll
-    for (int c = 0; c < NC; ++c) {
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            ck[c][e] = to_float<T>(rck[c].e[e]);
-            cv[c][e] = SHARED ? ck[c][e] : to_float<T>(rcv[c].e[e]);
-        }
-    }
+    // previous level's outputs (as floats, already rounded to the element type); the first level
+    // converts its children's pieces where it uses them, so that its first parents do not wait
+    // for the last rows
+    float lk[NC / 2][VEC];
 #pragma unroll
     for (int j = 1; j <= TL; ++j) {
         const int np = NC >> j;
@@ -242,19 +219,28 @@ build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename 
 #pragma unroll
         for (int i = 0; i < NC / 2; ++i) {
             if (i < np) {
-                float fq[VEC], fk[VEC], fv[VEC];
+                float fq[VEC], fk[VEC], fv[VEC], k0[VEC], k1[VEC], v0[VEC], v1[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     fq[e] = to_float<T>(rq[base + i].e[e]);
                     fk[e] = to_float<T>(rk[base + i].e[e]);
                     fv[e] = to_float<T>(rv[base + i].e[e]);
+                    if (j == 1) {
+                        k0[e] = to_float<T>(rck[2 * i].e[e]);
+                        k1[e] = to_float<T>(rck[2 * i + 1].e[e]);
+                        v0[e] = SHARED ? k0[e] : to_float<T>(rcv[SHARED ? 0 : 2 * i].e[e]);
+                        v1[e] = SHARED ? k1[e] : to_float<T>(rcv[SHARED ? 0 : 2 * i + 1].e[e]);
+                    } else {
+                        k0[e] = v0[e] = lk[2 * i][e];
+                        k1[e] = v1[e] = lk[2 * i + 1][e];
+                    }
                 }
                 float s0 = 0.f, s1 = 0.f, s2 = 0.f;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     s0 = fmaf(fq[e], fk[e], s0);
-                    s1 = fmaf(fq[e], ck[2 * i][e], s1);
-                    s2 = fmaf(fq[e], ck[2 * i + 1][e], s2);
+                    s1 = fmaf(fq[e], k0[e], s1);
+                    s2 = fmaf(fq[e], k1[e], s2);
                 }
                 if (!dok) { s0 = 0.f; s1 = 0.f; s2 = 0.f; }
                 s0 = group_sum(s0, G);
@@ -265,7 +251,7 @@ build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename 
                 float r[VEC];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
-                    float x = w0 * fv[e] + w1 * cv[2 * i][e] + w2 * cv[2 * i + 1][e];
+                    float x = w0 * fv[e] + w1 * v0[e] + w2 * v1[e];
                     r[e] = to_float<T>(from_float<T>(x));  // the stored value feeds the next level
                 }
                 if (active && dok) {
@@ -273,7 +259,7 @@ build_subtree_kernel(const typename T::storage *__restrict__ Qp, const typename 
                     if (o2) store_vec<T, VEC>(o2 + (size_t)i * rs, r);
                 }
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) { ck[i][e] = r[e]; cv[i][e] = r[e]; }
+                for (int e = 0; e < VEC; ++e) lk[i][e] = r[e];
             }
         }
     }
@@ -533,9 +519,19 @@ int build_parents_dispatch(const void *qp, const void *kp, const void *vp, const
     return build_parents_strided(qp, kp, vp, kc, vc, out, out2, weights, B, P, H, D, sd, dtype, st);
 }
 
+int build_tree_fused_dispatch(const void *qp, const void *kp, const void *vp, const void *k_leaf, const void *v_leaf,
+                              void *out, void *out2, int B, int N, int H, int D, int64_t qp_bs, int64_t kp_bs,
+                              int64_t vp_bs, int64_t kleaf_bs, int64_t vleaf_bs, int64_t out_bs, int64_t out2_bs,
+                              int dtype, hipStream_t st);  // hsa_build_tree.hip
+int build_tree_tune(int mode, int threads);
+
 }  // namespace hsa
 
 extern "C" {
+
+int hsa_build_tree_tune(int mode, int workgroup_threads) {
+    return hsa::build_tree_tune(mode, workgroup_threads);
+}
 
 int hsa_build_parents_fwd(const void *qp, const void *kp, const void *vp, const void *kc,
                           const void *vc, void *out, void *weights, int B, int P, int H, int D,
@@ -579,6 +575,13 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
     if (!kleaf_bs) kleaf_bs = leaf;
     if (!vleaf_bs) vleaf_bs = leaf;
     HSA_REQUIRE(dtype == HSA_F32 || dtype == HSA_F16 || dtype == HSA_BF16, "unknown dtype %d", dtype);
+    {
+        // one launch for the whole tree where the shape, the stream and the counter pool allow it
+        int rc = hsa::build_tree_fused_dispatch(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs,
+                                                vp_bs, kleaf_bs, vleaf_bs, out_bs, out2_bs, dtype,
+                                                (hipStream_t)stream);
+        if (rc != HSA_ERR_UNSUPPORTED) return rc;
+    }
     {
         int rc = hsa::build_tree_dispatch(qp, kp, vp, k_leaf, v_leaf, out, out2, B, N, H, D, qp_bs, kp_bs, vp_bs,
                                           kleaf_bs, vleaf_bs, out_bs, out2_bs, dtype, (hipStream_t)stream);

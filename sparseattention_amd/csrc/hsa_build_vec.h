@@ -1,0 +1,65 @@
+// 16-byte (or scalar) row pieces shared by the parent-build kernels.
+#pragma once
+#include "hsa_common.h"
+
+namespace hsa {
+
+template <typename T, int VEC> struct Pack { typename T::storage e[VEC]; };
+
+template <typename T, int VEC>
+__device__ __forceinline__ void load_vec(const typename T::storage *p, float (&f)[VEC]) {
+    if constexpr (VEC == 1) {
+        f[0] = to_float<T>(p[0]);
+    } else {
+        using P = Pack<T, VEC>;
+        P v = *reinterpret_cast<const P *>(p);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) f[i] = to_float<T>(v.e[i]);
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_vec(typename T::storage *p, const float (&f)[VEC]) {
+    if constexpr (VEC == 1) {
+        p[0] = from_float<T>(f[0]);
+    } else {
+        using P = Pack<T, VEC>;
+        P v;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v.e[i] = from_float<T>(f[i]);
+        static_assert(sizeof(P) == 16, "vector path moves 16 bytes per lane");
+        // regular store: the rows are read again by the next launch (a streaming store makes the
+        // tree build itself ~8% faster and the attention kernel after it as much slower)
+        *reinterpret_cast<P *>(p) = v;
+    }
+}
+
+// 16-byte load of a row piece that is read once per launch (streaming hint), as a Pack-like P
+#ifndef HSA_TREE_NT
+#define HSA_TREE_NT 1
+#endif
+template <typename P> __device__ __forceinline__ P load_once(const void *p) {
+    if constexpr (sizeof(P) == 16 && HSA_TREE_NT) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        const u4 v = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p));
+        return __builtin_bit_cast(P, v);
+    } else {
+        return *reinterpret_cast<const P *>(p);
+    }
+}
+
+// 16-byte store of a node row piece; WHICH = 0 for the first output, 1 for the second copy.
+// HSA_TREE_NTS bit WHICH selects the streaming hint for that output.
+#ifndef HSA_TREE_NTS
+#define HSA_TREE_NTS 0
+#endif
+template <int WHICH, typename P> __device__ __forceinline__ void store_node(void *p, const P &v) {
+    if constexpr (sizeof(P) == 16 && ((HSA_TREE_NTS >> WHICH) & 1)) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(p));
+    } else {
+        *reinterpret_cast<P *>(p) = v;
+    }
+}
+
+}  // namespace hsa

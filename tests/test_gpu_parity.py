@@ -341,6 +341,75 @@ def test_build_tree_vs_oracle(N, H, D, dtype):
     assert torch.equal(kfull[:, :N], kl.to(DEV)) and not vfull[:, :N].any()
 
 
+@pytest.fixture
+def tree_knobs():
+    """Sets how hsa_build_tree_fwd runs for one test and restores the defaults."""
+    from sparseattention_amd import _lib
+
+    def set_knobs(single_launch, threads):
+        assert _lib.lib().hsa_build_tree_tune(single_launch, threads) == 0
+    yield set_knobs
+    assert _lib.lib().hsa_build_tree_tune(1, 0) == 0
+
+
+# shapes chosen so that the single launch finishes 0..4 levels inside a workgroup and closes the
+# rest in one, two or several rounds of "last workgroup to arrive" (N=16384 with 16 heads of 128:
+# two subtrees per workgroup, four rounds)
+FUSED_TREE_CASES = [(2, 8, 8, 64), (3, 64, 8, 64), (2, 512, 8, 64), (8, 2048, 8, 64), (1, 16384, 16, 128),
+                    (2, 1024, 2, 64), (2, 256, 1, 32), (1, 4096, 4, 128), (2, 2048, 16, 64), (1, 8192, 8, 32)]
+
+
+@pytest.mark.parametrize("case", FUSED_TREE_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("threads", [0, 64, 128, 256, 512])
+def test_build_tree_single_launch(case, dtype, threads, tree_knobs):
+    """The whole tree in one launch against the oracle and against the multi-launch path, for
+    every workgroup size; run twice on the same buffers (the arrival counters must be back at
+    zero after a launch)."""
+    B, N, H, D = case
+    g = torch.Generator().manual_seed(N + H)
+    qp, kp, vp = (torch.randn(B, N - 1, H, D, generator=g).to(dtype).to(DEV) for _ in range(3))
+    kl, vl = (torch.randn(B, N, H, D, generator=g).to(dtype).to(DEV) for _ in range(2))
+    tree_knobs(0, -1)
+    stepwise = sa.build_tree(qp, kp, vp, kl, vl)
+    tree_knobs(2, threads)
+    out2 = torch.empty_like(stepwise)
+    fused = sa.build_tree(qp, kp, vp, kl, vl, out2=out2)
+    again = sa.build_tree(qp, kp, vp, kl, vl)
+    assert torch.equal(fused, again) and torch.equal(fused, out2)
+    want = oracle.build_tree_ref(qp.cpu(), kp.cpu(), vp.cpu(), kl.cpu(), vl.cpu(), compute_dtype=torch.float64)
+    assert_close(fused, want, dtype, "single launch")
+    # same arithmetic in both paths: they may differ by the rounding of one fused multiply-add
+    atol = 1e-6 if dtype == torch.float32 else 2e-2
+    assert (fused.float() - stepwise.float()).abs().max() <= atol
+
+
+def test_build_tree_single_launch_on_concurrent_streams(tree_knobs):
+    """Launches on different streams overlap on the GPU and must not share arrival counters:
+    four streams each build their own tree several times while the others run."""
+    tree_knobs(2, 512)
+    B, N, H, D = 4, 2048, 8, 64
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    data, outs = [], []
+    for i in range(4):
+        g = torch.Generator().manual_seed(100 + i)
+        data.append([torch.randn(B, rows, H, D, generator=g).to(torch.bfloat16).to(DEV)
+                     for rows in (N - 1, N - 1, N - 1, N, N)])
+        outs.append([torch.empty(B, N - 1, H, D, dtype=torch.bfloat16, device=DEV) for _ in range(6)])
+    torch.cuda.synchronize()
+    for rep in range(6):
+        for i, st in enumerate(streams):
+            with torch.cuda.stream(st):
+                sa.build_tree(*data[i], out=outs[i][rep])
+    torch.cuda.synchronize()
+    tree_knobs(0, -1)
+    for i in range(4):
+        want = sa.build_tree(*data[i])
+        for rep in range(6):
+            assert (outs[i][rep].float() - want.float()).abs().max() <= 2e-2, "stream %d repetition %d" % (i, rep)
+            assert torch.equal(outs[i][rep], outs[i][0])
+
+
 # ---------------------------------------------------------------- initial span nodes
 @pytest.mark.parametrize("shape", [(2, 2, 8), (1, 64, 48), (2, 4096, 512), (1, 128, 7)])
 @pytest.mark.parametrize("dtype", DTYPES)
