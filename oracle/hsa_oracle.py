@@ -138,7 +138,7 @@ def topology_scalar(seq_len: int) -> Tuple[np.ndarray, np.ndarray]:
 def attention_ref(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
                   idx_table, mask_table=None, window_size: int = 16,
                   compute_dtype: Optional[torch.dtype] = None,
-                  return_weights: bool = False, chunk: int = 4096):
+                  return_weights: bool = False, chunk: int = 4096, query_range=None):
     """Gather + einsum + softmax form of the leaf update.
 
     Follows hierarchical_attention_project/Hierarchical_Attention_Triton_Test.py:277-337
@@ -150,6 +150,8 @@ def attention_ref(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
     mask_table [N,L] bool or None.  Returns Out [B,N,H,D] in `compute_dtype`
     (default: Q's dtype, which reproduces the reference's stage-wise rounding),
     and optionally Weights [B,N,H,2R+1+L] (window slots first, then levels).
+    `query_range=(lo, hi)` evaluates only queries lo..hi-1 (the other output rows are left
+    uninitialised): a bounded sample for timing long sequences.
     """
     B, N, H, D = Q.shape
     R = int(window_size)
@@ -165,8 +167,9 @@ def attention_ref(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
     out = torch.empty(B, H, N, D, dtype=dt)
     wts = torch.empty(B, H, N, 2 * R + 1 + Lv, dtype=dt) if return_weights else None
     offs = torch.arange(-R, R + 1)
-    for s in range(0, N, chunk):
-        e = min(N, s + chunk)
+    q_lo, q_hi = query_range if query_range is not None else (0, N)
+    for s in range(q_lo, q_hi, chunk):
+        e = min(q_hi, s + chunk)
         rows = torch.arange(s, e).unsqueeze(1)
         swa = rows + offs.unsqueeze(0)                      # [n, 2R+1]
         valid = (swa >= 0) & (swa < N)

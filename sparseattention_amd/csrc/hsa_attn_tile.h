@@ -46,13 +46,16 @@ constexpr float NEG_INF = -__builtin_inff();
 
 // Which global accesses carry the streaming (non-temporal) hint, as a bit set: 1 = query rows,
 // 2 / 16 = the key / value leaf block that enters per query block, 8 = the leaf blocks carried
-// into a strip, 4 = tree nodes, 32 = plain instead of streaming output stores.  Query rows
-// and output rows are touched once per launch; marking them (and only them) as streaming
-// leaves the caches to the rows that neighbouring strips share: headline shape 17.6 us
-// against 20.2 us without the hint on the query loads (streaming loads on the key / value
-// rows as well: 18.8 - 19.7 us; plain output stores: 22.8 us).
+// into a strip, 4 = tree nodes, 32 = plain instead of streaming output stores.  Rows that one
+// wavefront touches once per launch (queries, entering leaf blocks, output) are marked; rows
+// that neighbouring strips share (carried-in blocks, tree nodes) stay cacheable.  Measured on
+// the headline shape with inputs rotated through 1.2 GB (nothing cache-resident): 20.6 us with
+// 1|2|16, 20.8 us with 1 alone or none of the load hints, 21.1 us with every load marked; plain
+// output stores cost 2.5 us.  (With only 400 MB rotated the hint on the query rows alone looks
+// like 12 %: it keeps them out of the 256 MB memory-side cache, which then holds more of the
+// other tensors -- an artefact of too small a rotation, not a property of the kernel.)
 #ifndef HSA_TILE_NT
-#define HSA_TILE_NT 1
+#define HSA_TILE_NT 19
 #endif
 // 16-byte global load, optionally with the streaming (non-temporal) hint
 template <bool NT> __device__ __forceinline__ u32x4_t ld16(const uint16_t *p) {
@@ -292,18 +295,30 @@ attn_tile_kernel(TileParams p) {
     // requests run AHEAD blocks in front of the computation
     constexpr int AHEAD = (D <= 64) ? 2 : 1;
     Stage st[SB];
+
+    // ---- per-strip operands: far tree block, leaf blocks carried into the first query block ----
+    // Everything the strip's first block needs is requested before anything is consumed, in
+    // the order of use (loads return in order): one memory round trip for the prologue.
+    u32x4_t far_k[NLD], far_v[NLD];
+    load_far(Kb, far_k);
+    load_far(Vb, far_v);
+    u32x4_t halo_k[NKL][NLD], halo_v[NKL][NLD];
+#pragma unroll
+    for (int c = 0; c < NKL; ++c) {
+        if (c == NEWI) continue;
+        const int row0 = leaf_row0(seq(0) - NBW + c);
+        load_block(Kb, row0, halo_k[c], nt_halo);
+        load_block(Vb, row0, halo_v[c], nt_halo);
+    }
 #pragma unroll
     for (int i = 0; i < AHEAD && i < SB; ++i) request(st[i], seq(i));
 
-    // ---- per-strip operands: far tree block, leaf blocks carried into the first query block ----
     u32x4_t Ku[KS];
     u32x2_t Vu[NJ];
     {
-        u32x4_t rk[NLD], rv[NLD], vop[KS];
-        load_far(Kb, rk);
-        load_far(Vb, rv);
-        lds_put(0, rk);
-        lds_put(1, rv);
+        u32x4_t vop[KS];
+        lds_put(0, far_k);
+        lds_put(1, far_v);
         lds_get(0, Ku);
         lds_get(1, vop);
         transpose_v(vop, Vu);
@@ -313,12 +328,9 @@ attn_tile_kernel(TileParams p) {
 #pragma unroll
     for (int c = 0; c < NKL; ++c) {
         if (c == NEWI) continue;
-        const int row0 = leaf_row0(seq(0) - NBW + c);
-        u32x4_t rk[NLD], rv[NLD], vop[KS];
-        load_block(Kb, row0, rk, nt_halo);
-        load_block(Vb, row0, rv, nt_halo);
-        lds_put(2, rk);
-        lds_put(3, rv);
+        u32x4_t vop[KS];
+        lds_put(2, halo_k[c]);
+        lds_put(3, halo_v[c]);
         lds_get(2, Kl[c]);
         lds_get(3, vop);
         transpose_v(vop, Vl[c]);
