@@ -66,8 +66,9 @@ const char *hsa_last_error(void);
  *   causal      used only when idx == NULL
  *   dtype       HSA_F32 / HSA_F16 / HSA_BF16
  *   algo        HSA_ATTN_*.  The MFMA tile kernels take canonical tables (idx == NULL), no
- *               weights, R <= 32, 16 <= N <= 2^22, and head sizes 32 / 64 / 128 for the
- *               16-bit types, 32 / 64 for fp32; everything else runs on the gather kernel
+ *               weights, 16 <= N <= 2^22, R <= 32 (16-bit types, causal: R <= 64), and head
+ *               sizes 32 / 64 / 128 for the 16-bit types, 32 / 64 for fp32; everything else
+ *               runs on the gather kernel
  */
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
@@ -101,7 +102,9 @@ int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_
  */
 int hsa_attn_tile_tune(int strip_blocks, int waves_per_group, int xcd_remap, int alternate);
 
-/* 1 if HSA_ATTN_AUTO would pick the MFMA tile kernel for this problem, else 0. */
+/* 1 if HSA_ATTN_AUTO would pick the MFMA tile kernel for this problem, else 0.
+ * canonical_tables: 0 = tables given explicitly, 1 = canonical tables, not causal,
+ * 2 = canonical tables, causal (the causal kernels take a larger window radius). */
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype,
                            int canonical_tables, int want_weights);
 

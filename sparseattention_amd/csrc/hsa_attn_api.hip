@@ -8,7 +8,7 @@ int attn_gather_dispatch(const void *q, const void *k, const void *v, const int3
                          int D, int L, int R, int causal, int dtype, hipStream_t st);
 
 bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
-                        bool want_weights);
+                        bool want_weights, bool causal);
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st);
 int attn_tile_tune(int sb, int wpb, int swizzle, int alternate);
@@ -17,9 +17,10 @@ int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *ou
                            int D, int L, int R, int causal, hipStream_t st);
 
 // the MFMA tile kernels: 16-bit element types, or fp32 on the fp32 matrix instructions
-static bool tile_ok_for(int N, int M, int H, int D, int L, int R, int dtype, bool canonical, bool want_weights) {
+static bool tile_ok_for(int N, int M, int H, int D, int L, int R, int dtype, bool canonical, bool want_weights,
+                        bool causal) {
     if (dtype == HSA_F32) return attn_tile_f32_eligible(N, M, D, L, R, canonical, want_weights);
-    return attn_tile_eligible(N, M, H, D, L, R, dtype, canonical, want_weights);
+    return attn_tile_eligible(N, M, H, D, L, R, dtype, canonical, want_weights, causal);
 }
 
 }  // namespace hsa
@@ -32,7 +33,8 @@ int hsa_attn_tile_tune(int strip_blocks, int waves_per_group, int xcd_remap, int
 
 int hsa_attn_fwd_uses_tile(int N, int M, int H, int D, int L, int R, int dtype, int canonical_tables,
                            int want_weights) {
-    return hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical_tables != 0, want_weights != 0) ? 1 : 0;
+    return hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical_tables != 0, want_weights != 0,
+                            canonical_tables == 2) ? 1 : 0;
 }
 
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
@@ -52,7 +54,7 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
         causal = (mask != nullptr);
     }
     hipStream_t st = (hipStream_t)stream;
-    bool tile_ok = hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical, weights != nullptr);
+    bool tile_ok = hsa::tile_ok_for(N, M, H, D, L, R, dtype, canonical, weights != nullptr, causal != 0);
     // the tile kernels move 16-byte pieces: tensors at other addresses (a view at an odd element
     // offset) go to the gather kernel unless the tile kernel was asked for by name
     const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0;

@@ -66,6 +66,7 @@ template <bool NT> __device__ __forceinline__ u32x4_t ld16(const uint16_t *p) {
 struct TileParams {
     const uint16_t *q, *k, *v;
     uint16_t *out;
+    float *weights;  // [B, N, H, 2R+1+L] or null (kernels built with WT only)
     int B, N, M, H, L, R;
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
@@ -88,7 +89,11 @@ template <int D> constexpr int tile_max_wpb() { return D > 64 ? 4 : 8; }
 // 19.5 us against 23.4 us).  Each wavefront re-lays the 16-byte pieces out into MFMA operand
 // order through a private, padded LDS region (no workgroup barrier: a wavefront's LDS
 // operations execute in order), and the output takes the reverse route.
-template <typename T, int D, int NBW, bool CAUSAL, int SB>
+// WT: also write the fp32 softmax weights [B, N, H, 2R+1+L] (window slots first, then levels;
+// dead slots zero).  A block's 16 rows of weights are assembled in the wavefront's LDS region
+// (the operand slots are free once the MFMA operands have been read) and written out as
+// whole rows.  Needs 2R+1+L <= D*2+16 floats per row to fit.
+template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false>
 __global__ void __launch_bounds__(tile_max_wpb<D>() * 64)
 attn_tile_kernel(TileParams p) {
     using M_ = Mma<T>;
@@ -405,6 +410,7 @@ attn_tile_kernel(TileParams p) {
 
         float den = 0.f;
         u32x2_t P[NKL + 2];
+        float ew[WT ? NKL + 2 : 1][4];
 #pragma unroll
         for (int c = 0; c < NKL + 2; ++c) {
             float e[4];
@@ -412,12 +418,51 @@ attn_tile_kernel(TileParams p) {
             for (int i = 0; i < 4; ++i) {
                 e[i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
                 den += e[i];
+                if constexpr (WT) ew[c][i] = e[i];
             }
             P[c] = u32x2_t{M_::pack(e[0], e[1]), M_::pack(e[2], e[3])};
         }
         den += __shfl_xor(den, 16, 64);
         den += __shfl_xor(den, 32, 64);
         const float inv = 1.0f / den;
+
+        if constexpr (WT) {
+            // rows of weights in LDS: query r of the block at float offset r * S, in operand slots 1..4
+            const int S = 2 * R + 1 + L;
+            float *wrow = reinterpret_cast<float *>(lds + BLK_BYTES);
+            for (int t = lane; t < TILE_Q * S; t += 64) wrow[t] = 0.f;
+            __builtin_amdgcn_wave_barrier();
+            float *mine = wrow + r16 * S;
+#pragma unroll
+            for (int c = 0; c < NKL; ++c) {
+                const int kb = blk - NBW + c;
+                if (kb < 0 || kb >= NB) continue;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int kl = 4 * g + i;
+                    const int diff = TILE_Q * (c - NBW) + kl - r16;  // key row - query row
+                    const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+                    const bool sib = c == NBW && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
+                    // a key that is both a window slot and the level-0 neighbour carries twice the weight
+                    const float w = ew[c][i] * inv * ((win && sib) ? 0.5f : 1.0f);
+                    if (win) mine[diff + R] = w;
+                    if (sib) mine[2 * R + 1] = w;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int sl = 4 * g + i;
+                const int lvl = sl < 8 ? 1 : (sl < 12 ? 2 : (sl < 14 ? 3 : 4 + (sl - 14)));
+                if (sc[NKL][i] > NEG_INF) mine[2 * R + 1 + lvl] = ew[NKL][i] * inv;
+                const int ul = 6 + sl;
+                if (sc[NKL + 1][i] > NEG_INF) mine[2 * R + 1 + ul] = ew[NKL + 1][i] * inv;
+            }
+            __builtin_amdgcn_wave_barrier();
+            float *wg_out = p.weights + (((size_t)b * N + q0) * p.H + h) * S;
+            for (int r = 0; r < TILE_Q; ++r)
+                for (int t = lane; t < S; t += 64) wg_out[(size_t)r * p.H * S + t] = wrow[r * S + t];
+            __builtin_amdgcn_wave_barrier();
+        }
 
         // O^T tiles: this lane ends with channels [32ks + 8g, +8) of query r16; through LDS
         // back to whole rows, then streaming stores (the output is not read again here)
@@ -482,5 +527,8 @@ attn_tile_kernel(TileParams p) {
 
 template <typename T, int D>
 int attn_tile_launch_td(const TileParams &p, int nbw, bool causal, int sb, int wpb, hipStream_t st);
+// the variant that also writes the softmax weights (one query block per wavefront)
+template <typename T, int D>
+int attn_tile_weights_launch_td(const TileParams &p, int nbw, bool causal, int wpb, hipStream_t st);
 
 }  // namespace hsa

@@ -7,6 +7,9 @@
 
 namespace hsa {
 
+// window radius in 16-row leaf blocks: up to 4 (R <= 64) when causal, where a query block sees
+// NBW + 1 leaf blocks; up to 2 (R <= 32) otherwise, where it sees 2 NBW + 1
+constexpr int TILE_MAX_NBW_CAUSAL = 4;
 constexpr int TILE_MAX_NBW = 2;
 
 // Experiment knobs of the tile launch: strip length in query blocks (0 = by problem size),
@@ -45,25 +48,28 @@ int attn_tile_tune(int sb, int wpb, int swizzle, int alternate) {
 }
 
 bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
-                        bool want_weights) {
+                        bool want_weights, bool causal) {
     (void)H;
-    if (!canonical || want_weights) return false;
+    if (!canonical) return false;
+    // the weights of a query block are assembled in the wavefront's LDS region: a row of
+    // 2R+1+L floats has to fit the operand pitch
+    if (want_weights && 2 * R + 1 + L > D * 2 + 16) return false;
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS) return false;
     if (M < 2 * N - 1) return false;
-    if ((R + TILE_Q - 1) / TILE_Q > TILE_MAX_NBW) return false;
+    if ((R + TILE_Q - 1) / TILE_Q > (causal ? TILE_MAX_NBW_CAUSAL : TILE_MAX_NBW)) return false;
     return true;
 }
 
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st) {
-    (void)weights;
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
         return fail(HSA_ERR_INVALID, "tile kernel needs 16-byte aligned tensors");
     TileParams p;
     p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v;
     p.out = (uint16_t *)out;
+    p.weights = weights;
     p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
     const int NB = N / TILE_Q;
     TileKnobs &knobs = tile_knobs();
@@ -72,7 +78,9 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     const long block_units = (long)B * H * NB;
     int sb = block_units >= 4 * 2048 ? 4 : (block_units >= 2 * 2048 ? 2 : 1);
     if (const int forced = knobs.sb) sb = forced;
-    if (!causal && (R + TILE_Q - 1) / TILE_Q >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
+    // four or five leaf blocks per query block: shorter strips keep the operands in registers
+    if ((R + TILE_Q - 1) / TILE_Q >= (causal ? 3 : 2) && sb > 2) sb = 2;
+    if ((R + TILE_Q - 1) / TILE_Q >= 4 && !knobs.sb) sb = 1;  // longer strips spill at five leaf blocks + halo
     while (sb > NB) sb >>= 1;  // NB is a power of two
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;
@@ -83,6 +91,21 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
     const int wpb = knobs.wpb;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
+    if (weights) {
+        // one query block per wavefront
+        p.NS = NB;
+        const long wunits = (long)B * NB * H;
+        if (wunits > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+        p.n_units = (int)wunits;
+        if (dtype == HSA_BF16) {
+            if (D == 32) return attn_tile_weights_launch_td<BF16, 32>(p, nbw, causal != 0, wpb, st);
+            if (D == 64) return attn_tile_weights_launch_td<BF16, 64>(p, nbw, causal != 0, wpb, st);
+            return attn_tile_weights_launch_td<BF16, 128>(p, nbw, causal != 0, wpb, st);
+        }
+        if (D == 32) return attn_tile_weights_launch_td<F16, 32>(p, nbw, causal != 0, wpb, st);
+        if (D == 64) return attn_tile_weights_launch_td<F16, 64>(p, nbw, causal != 0, wpb, st);
+        return attn_tile_weights_launch_td<F16, 128>(p, nbw, causal != 0, wpb, st);
+    }
     if (dtype == HSA_BF16) {
         if (D == 32) return attn_tile_launch_td<BF16, 32>(p, nbw, causal != 0, sb, wpb, st);
         if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, sb, wpb, st);

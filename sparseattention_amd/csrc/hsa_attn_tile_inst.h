@@ -21,6 +21,14 @@ static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
 }
 
 template <typename T, int D, int NBW, bool CAUSAL>
+static int tile_launch_weights(const TileParams &p, int wpb, hipStream_t st) {
+    if (wpb > tile_max_wpb<D>()) wpb = tile_max_wpb<D>();
+    const int nwg = (p.n_units + wpb - 1) / wpb;
+    attn_tile_kernel<T, D, NBW, CAUSAL, 1, true><<<nwg, wpb * 64, 0, st>>>(p);
+    return check_launch("attn_tile_kernel (weights)");
+}
+
+template <typename T, int D, int NBW, bool CAUSAL>
 static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) {
     switch (sb) {
         case 1: return tile_launch_one<T, D, NBW, CAUSAL, 1>(p, wpb, st);
@@ -41,6 +49,23 @@ static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) 
             case 3: return tile_launch_sb<T, D, 1, true>(p, sb, wpb, st);                       \
             case 4: return tile_launch_sb<T, D, 2, false>(p, sb, wpb, st);                      \
             case 5: return tile_launch_sb<T, D, 2, true>(p, sb, wpb, st);                       \
+            case 7: return tile_launch_sb<T, D, 3, true>(p, sb, wpb, st);                       \
+            case 9: return tile_launch_sb<T, D, 4, true>(p, sb, wpb, st);                       \
+        }                                                                                       \
+        return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel");       \
+    }                                                                                           \
+    template <>                                                                                 \
+    int attn_tile_weights_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int wpb,  \
+                                          hipStream_t st) {                                     \
+        switch (nbw * 2 + (causal ? 1 : 0)) {                                                   \
+            case 0: return tile_launch_weights<T, D, 0, false>(p, wpb, st);                     \
+            case 1: return tile_launch_weights<T, D, 0, true>(p, wpb, st);                      \
+            case 2: return tile_launch_weights<T, D, 1, false>(p, wpb, st);                     \
+            case 3: return tile_launch_weights<T, D, 1, true>(p, wpb, st);                      \
+            case 4: return tile_launch_weights<T, D, 2, false>(p, wpb, st);                     \
+            case 5: return tile_launch_weights<T, D, 2, true>(p, wpb, st);                      \
+            case 7: return tile_launch_weights<T, D, 3, true>(p, wpb, st);                      \
+            case 9: return tile_launch_weights<T, D, 4, true>(p, wpb, st);                      \
         }                                                                                       \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel");       \
     }

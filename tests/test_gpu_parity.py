@@ -514,6 +514,32 @@ TILE_CASES = [  # B, N, H, D, R
     (1, 64, 3, 32, 20),
     (1, 1024, 8, 32, 16),
 ]
+# causal only: window radius above 32 (four or five leaf blocks per query block)
+TILE_CASES_WIDE = [(2, 256, 4, 64, 48), (1, 512, 2, 64, 64), (1, 128, 2, 128, 50), (2, 256, 3, 32, 64), (1, 64, 2, 64, 33)]
+
+
+@pytest.mark.parametrize("case", TILE_CASES_WIDE)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("strip", [None, "1", "2"])
+def test_attention_tile_wide_causal_window(case, dtype, strip, tile_knobs):
+    """Causal windows of radius 33..64 stay on the tile kernel; the same radius without the causal
+    mask is refused by it (and served by the gather kernel under the automatic choice)."""
+    B, N, H, D, R = case
+    if strip is not None:
+        tile_knobs(int(strip), -1, -1, -1)
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
+    t = sa.build_tree_topology(N, True, device=DEV)
+    o = oracle.topology_tables(N, True)
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], t["forward_mask"], R, algo="tile")
+    want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"], R, compute_dtype=torch.float64)
+    assert_close(out, want, dtype, "tile, wide causal window")
+    tn = sa.build_tree_topology(N, False, device=DEV)
+    with pytest.raises(sa.HsaError):
+        fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
+    on = oracle.topology_tables(N, False)
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R)
+    want = oracle.attention_ref(q, k, v, on["forward_idx"], None, R, compute_dtype=torch.float64)
+    assert_close(out, want, dtype, "automatic choice, wide window, not causal")
 
 
 @pytest.mark.parametrize("case", TILE_CASES)
@@ -534,6 +560,37 @@ def test_attention_tile_vs_oracle(case, dtype, causal, strip, tile_knobs):
     want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
                                 compute_dtype=torch.float64)
     assert_close(out, want, dtype, "tile")
+
+
+@pytest.mark.parametrize("case", TILE_CASES + [(1, 256, 2, 64, 48), (1, 64, 2, 32, 24)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_tile_weights_vs_oracle(case, dtype, causal):
+    """The tile kernel's softmax weights [B, N, H, 2R+1+L] (fp32; window slots first, then one
+    per level; dead slots zero; the sibling leaf's weight split over its two slots) and its
+    output, against the oracle; every row of weights sums to one."""
+    B, N, H, D, R = case
+    if not causal and R > 32:
+        pytest.skip("the tile kernel takes a window radius above 32 only when causal")
+    L = N.bit_length() - 1
+    if 2 * R + 1 + L > 2 * D + 16:
+        pytest.skip("a row of weights does not fit the wavefront's staging area")
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    o = oracle.topology_tables(N, causal)
+    out, w = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                                  t["forward_mask"] if causal else None, R, return_weights=True, algo="tile")
+    want, want_w = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
+                                        compute_dtype=torch.float64, return_weights=True)
+    assert w.dtype == torch.float32 and w.shape == (B, N, H, 2 * R + 1 + L)
+    assert_close(out, want, dtype, "tile output with weights")
+    assert (w.double().cpu() - want_w).abs().max() < 2e-5
+    assert (w.sum(-1) - 1).abs().max() < 1e-5
+    assert ((want_w == 0) <= (w.cpu() == 0)).all()      # dead slots are exact zeros
+    # the gather kernel's weights agree
+    _, wg = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                                 t["forward_mask"] if causal else None, R, return_weights=True, algo="gather")
+    assert (w - wg).abs().max() < 2e-5
 
 
 @pytest.mark.parametrize("seed", range(24))
