@@ -244,6 +244,25 @@ int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, cons
                           void *dvc, int B, int P, int H, int D, int dtype, void *stream);
 
 /*
+ * hsa_build_parents_bwd on operands that are column slices of wider matrices: the backward of the
+ * level step of HierarchicalAttention.cross_update_Y
+ * (hierarchical_attention/modules/attention.py:119-157; the reference differentiates it through
+ * BuildParentNodesFunc.backward, ops/functional.py:66-111, and the autograd of its Linear layers)
+ * when the projections that feed the level are fused: q/k/v of the parents are thirds of one
+ * [B, N-1, 3*H*D] projection, the children's k/v halves of one [B, 2P, 2*H*D] projection, and
+ * their gradients are written into buffers of the same shapes (which the fused weight-gradient
+ * and input-gradient GEMMs then read whole).
+ *   batch_strides, row_strides   host arrays of 11 element counts in the order dout, qp, kp, vp,
+ *                                kc, vc, dqp, dkp, dvp, dkc, dvc; an entry of 0, or a NULL array,
+ *                                means dense
+ */
+int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *kp, const void *vp,
+                                  const void *kc, const void *vc, void *dqp, void *dkp, void *dvp,
+                                  void *dkc, void *dvc, int B, int P, int H, int D,
+                                  const int64_t *batch_strides, const int64_t *row_strides, int dtype,
+                                  void *stream);
+
+/*
  * Backward of the span attention for the canonical tables.
  * Replaces HierarchicalAttentionFunc.backward and its five kernels
  * (hierarchical_attention/ops/functional.py:171-264,

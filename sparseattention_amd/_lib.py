@@ -60,6 +60,8 @@ def _declare(lib):
     lib.hsa_span_input_y.restype = I
     lib.hsa_build_parents_bwd.argtypes = [P] * 11 + [I] * 5 + [P]
     lib.hsa_build_parents_bwd.restype = I
+    lib.hsa_build_parents_strided_bwd.argtypes = [P] * 11 + [I] * 4 + [P, P, I, P]
+    lib.hsa_build_parents_strided_bwd.restype = I
     lib.hsa_attn_bwd_workspace_bytes.argtypes = [I] * 9
     lib.hsa_attn_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.hsa_attn_bwd.argtypes = [P] * 8 + [ctypes.c_size_t] + [I] * 10 + [P]

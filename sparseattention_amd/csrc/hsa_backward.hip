@@ -47,6 +47,13 @@ __device__ __forceinline__ void bstore(typename T::storage *p, const float (&f)[
     }
 }
 
+// Batch and row strides (in elements) of the eleven operands, in the order
+// dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc.
+struct BwdStrides {
+    int64_t bs[11];
+    int64_t rs[11];
+};
+
 template <typename T, int VEC, int CH>
 __global__ void __launch_bounds__(256)
 build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typename T::storage *__restrict__ Qp,
@@ -54,7 +61,8 @@ build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typen
                          const typename T::storage *__restrict__ Kc, const typename T::storage *__restrict__ Vc,
                          typename T::storage *__restrict__ dQ, typename T::storage *__restrict__ dKp,
                          typename T::storage *__restrict__ dVp, typename T::storage *__restrict__ dKc,
-                         typename T::storage *__restrict__ dVc, int B, int P, int H, int D, int G, float scale) {
+                         typename T::storage *__restrict__ dVc, int B, int P, int H, int D, int G, BwdStrides sd,
+                         float scale) {
     const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
     const long unit = tid / G;
     const int gl = (int)(tid % G);
@@ -64,9 +72,13 @@ build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typen
     const int h = (int)(u % H);
     const int i = (int)((u / H) % P);
     const int b = (int)(u / ((long)H * P));
-    const size_t prow = (((size_t)b * P + i) * H + h) * D;
-    const size_t c0row = (((size_t)b * 2 * P + 2 * i) * H + h) * D;
-    const size_t c1row = c0row + (size_t)H * D;
+    // element offset of this (batch, row, head) in operand o; children: rows 2i and 2i+1
+    auto at = [&](int o, int row) { return (size_t)b * sd.bs[o] + (size_t)row * sd.rs[o] + (size_t)h * D; };
+    dO += at(0, i); Qp += at(1, i); Kp += at(2, i); Vp += at(3, i);
+    dQ += at(6, i); dKp += at(7, i); dVp += at(8, i);
+    const typename T::storage *Kc1 = Kc + at(4, 2 * i + 1), *Vc1 = Vc + at(5, 2 * i + 1);
+    typename T::storage *dKc1 = dKc + at(9, 2 * i + 1), *dVc1 = dVc + at(10, 2 * i + 1);
+    Kc += at(4, 2 * i); Vc += at(5, 2 * i); dKc += at(9, 2 * i); dVc += at(10, 2 * i);
 
     float q[CH][VEC], kp[CH][VEC], k0[CH][VEC], k1[CH][VEC], vp[CH][VEC], v0[CH][VEC], v1[CH][VEC], g[CH][VEC];
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, p0 = 0.f, p1 = 0.f, p2 = 0.f;
@@ -74,14 +86,14 @@ build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typen
     for (int c = 0; c < CH; ++c) {
         const int d = (c * G + gl) * VEC;
         if (d < D) {
-            bload<T, VEC>(Qp + prow + d, q[c]);
-            bload<T, VEC>(Kp + prow + d, kp[c]);
-            bload<T, VEC>(Kc + c0row + d, k0[c]);
-            bload<T, VEC>(Kc + c1row + d, k1[c]);
-            bload<T, VEC>(Vp + prow + d, vp[c]);
-            bload<T, VEC>(Vc + c0row + d, v0[c]);
-            bload<T, VEC>(Vc + c1row + d, v1[c]);
-            bload<T, VEC>(dO + prow + d, g[c]);
+            bload<T, VEC>(Qp + d, q[c]);
+            bload<T, VEC>(Kp + d, kp[c]);
+            bload<T, VEC>(Kc + d, k0[c]);
+            bload<T, VEC>(Kc1 + d, k1[c]);
+            bload<T, VEC>(Vp + d, vp[c]);
+            bload<T, VEC>(Vc + d, v0[c]);
+            bload<T, VEC>(Vc1 + d, v1[c]);
+            bload<T, VEC>(dO + d, g[c]);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) {
                 s0 = fmaf(q[c][e], kp[c][e], s0);
@@ -110,25 +122,25 @@ build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typen
             float r[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = ds0 * kp[c][e] + ds1 * k0[c][e] + ds2 * k1[c][e];
-            bstore<T, VEC>(dQ + prow + d, r);
+            bstore<T, VEC>(dQ + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = ds0 * q[c][e];
-            bstore<T, VEC>(dKp + prow + d, r);
+            bstore<T, VEC>(dKp + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = ds1 * q[c][e];
-            bstore<T, VEC>(dKc + c0row + d, r);
+            bstore<T, VEC>(dKc + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = ds2 * q[c][e];
-            bstore<T, VEC>(dKc + c1row + d, r);
+            bstore<T, VEC>(dKc1 + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = w0 * g[c][e];
-            bstore<T, VEC>(dVp + prow + d, r);
+            bstore<T, VEC>(dVp + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = w1 * g[c][e];
-            bstore<T, VEC>(dVc + c0row + d, r);
+            bstore<T, VEC>(dVc + d, r);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) r[e] = w2 * g[c][e];
-            bstore<T, VEC>(dVc + c1row + d, r);
+            bstore<T, VEC>(dVc1 + d, r);
         }
     }
 }
@@ -136,13 +148,15 @@ build_parents_bwd_kernel(const typename T::storage *__restrict__ dO, const typen
 template <typename T>
 static int build_parents_bwd_typed(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
                                    const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B,
-                                   int P, int H, int D, hipStream_t st) {
+                                   int P, int H, int D, const BwdStrides &sd, hipStream_t st) {
     using S = typename T::storage;
     constexpr int VEC16 = 16 / (int)sizeof(S);
     const uintptr_t al = (uintptr_t)dout | (uintptr_t)qp | (uintptr_t)kp | (uintptr_t)vp | (uintptr_t)kc |
                          (uintptr_t)vc | (uintptr_t)dqp | (uintptr_t)dkp | (uintptr_t)dvp | (uintptr_t)dkc |
                          (uintptr_t)dvc;
-    const bool vec_ok = D % VEC16 == 0 && (al & 15) == 0;
+    int64_t strides = 0;
+    for (int o = 0; o < 11; ++o) strides |= sd.bs[o] | sd.rs[o];
+    const bool vec_ok = D % VEC16 == 0 && (al & 15) == 0 && (strides % VEC16) == 0;
     const int vec = vec_ok ? VEC16 : 1;
     const int chunks = (D + vec - 1) / vec;
     int G = 1;
@@ -155,7 +169,7 @@ static int build_parents_bwd_typed(const void *dout, const void *qp, const void 
 #define HSA_BWD(VECN, CHN)                                                                                  \
     build_parents_bwd_kernel<T, VECN, CHN><<<(unsigned)blocks, 256, 0, st>>>(                               \
         (const S *)dout, (const S *)qp, (const S *)kp, (const S *)vp, (const S *)kc, (const S *)vc, (S *)dqp, \
-        (S *)dkp, (S *)dvp, (S *)dkc, (S *)dvc, B, P, H, D, G, scale)
+        (S *)dkp, (S *)dvp, (S *)dkc, (S *)dvc, B, P, H, D, G, sd, scale)
     if (vec_ok) {
         if (CH == 1) HSA_BWD(VEC16, 1);
         else if (CH == 2) HSA_BWD(VEC16, 2);
@@ -673,18 +687,42 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
 
 extern "C" {
 
+static int build_parents_bwd_any(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
+                                 const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B, int P,
+                                 int H, int D, const int64_t *batch_strides, const int64_t *row_strides, int dtype,
+                                 void *stream) {
+    HSA_REQUIRE(dout && qp && kp && vp && kc && vc && dqp && dkp && dvp && dkc && dvc, "null pointer");
+    HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
+    hsa::BwdStrides sd;
+    for (int o = 0; o < 11; ++o) {
+        const bool child = o == 4 || o == 5 || o == 9 || o == 10;
+        sd.rs[o] = row_strides && row_strides[o] ? row_strides[o] : (int64_t)H * D;
+        HSA_REQUIRE(sd.rs[o] >= (int64_t)H * D, "row stride %lld below H*D", (long long)sd.rs[o]);
+        sd.bs[o] = batch_strides && batch_strides[o] ? batch_strides[o] : (child ? 2 : 1) * (int64_t)P * sd.rs[o];
+        HSA_REQUIRE(sd.bs[o] >= 0, "negative stride");
+    }
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case HSA_F32: return hsa::build_parents_bwd_typed<hsa::F32>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, sd, st);
+        case HSA_F16: return hsa::build_parents_bwd_typed<hsa::F16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, sd, st);
+        case HSA_BF16: return hsa::build_parents_bwd_typed<hsa::BF16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, sd, st);
+    }
+    return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
 int hsa_build_parents_bwd(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
                           const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B, int P,
                           int H, int D, int dtype, void *stream) {
-    HSA_REQUIRE(dout && qp && kp && vp && kc && vc && dqp && dkp && dvp && dkc && dvc, "null pointer");
-    HSA_REQUIRE(B >= 1 && P >= 1 && H >= 1 && D >= 1, "bad shape B=%d P=%d H=%d D=%d", B, P, H, D);
-    hipStream_t st = (hipStream_t)stream;
-    switch (dtype) {
-        case HSA_F32: return hsa::build_parents_bwd_typed<hsa::F32>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
-        case HSA_F16: return hsa::build_parents_bwd_typed<hsa::F16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
-        case HSA_BF16: return hsa::build_parents_bwd_typed<hsa::BF16>(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, st);
-    }
-    return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+    return build_parents_bwd_any(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, nullptr, nullptr,
+                                 dtype, stream);
+}
+
+int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *kp, const void *vp, const void *kc,
+                                  const void *vc, void *dqp, void *dkp, void *dvp, void *dkc, void *dvc, int B,
+                                  int P, int H, int D, const int64_t *batch_strides, const int64_t *row_strides,
+                                  int dtype, void *stream) {
+    return build_parents_bwd_any(dout, qp, kp, vp, kc, vc, dqp, dkp, dvp, dkc, dvc, B, P, H, D, batch_strides,
+                                 row_strides, dtype, stream);
 }
 
 size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo) {

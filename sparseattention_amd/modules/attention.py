@@ -28,6 +28,29 @@ def _level_sizes(n_leaves: int) -> List[int]:
     return sizes
 
 
+class _SpanLevels(torch.autograd.Function):
+    """The level loop of `HierarchicalAttention.cross_update_Y` (reference
+    hierarchical_attention/modules/attention.py:101-157, everything before out_proj_y) as one
+    differentiable function on fused projections.  The reference gets the same gradients from
+    autograd through 3 + 2L Linear layers and L `BuildParentNodesFunc`s (ops/functional.py:66-111)."""
+
+    @staticmethod
+    def forward(ctx, module, drop_p, x, y_in, wq, wk, wv):
+        y_new, kept = module._span_levels(x, y_in, keep=True, drop_p=drop_p)
+        ctx.module, ctx.kept = module, kept
+        ctx.in_dtypes = (x.dtype, y_in.dtype, wq.dtype)
+        return y_new
+
+    @staticmethod
+    def backward(ctx, dy):
+        dx, dy_in, dw = ctx.module._span_levels_backward(dy, ctx.kept)
+        ctx.kept = None
+        xd, yd, wd = ctx.in_dtypes
+        D = dx.shape[-1]
+        dw = dw.to(wd)
+        return None, None, dx.to(xd), dy_in.to(yd), dw[:D], dw[D:2 * D], dw[2 * D:]
+
+
 class HierarchicalAttention(nn.Module):
     def __init__(self, dim: int, num_heads: int, dropout: float = 0.1, window_size: int = 16):
         super().__init__()
@@ -53,6 +76,7 @@ class HierarchicalAttention(nn.Module):
         self.offsets: Optional[List[int]] = None
         self._fused = {}  # row-concatenated projection weights of the no-autograd path
         self.fuse_top_levels = True  # no-autograd path: the last levels in one launch where the shape allows
+        self.fused_training = True   # autograd path: fused projections and one backward kernel per level
 
     # -- helpers -------------------------------------------------------------
     def _get_lookup_table(self, L: int, is_causal: bool, device: torch.device):
@@ -118,19 +142,23 @@ class HierarchicalAttention(nn.Module):
         return any(t.requires_grad for t in tensors) or any(
             p.requires_grad for m in layers for p in m.parameters())
 
-    def _cross_update_Y_direct(self, x: torch.Tensor, y_in: torch.Tensor) -> torch.Tensor:
-        """cross_update_Y without autograd and without dropout: the three projections of the span
-        nodes are one GEMM, the key/value projections of each level's children another, and each
-        level's kernel reads its operands as column slices of those results.  Every level writes
-        twice: a dense [B, P, D] block that feeds the next level's GEMM, and its slice of the
-        level-concatenated [B, N-1, D] result.  The last levels (few rows each) run as one
-        launch that does their projections on chip."""
+    def _span_levels(self, x: torch.Tensor, y_in: torch.Tensor, keep: bool = False, drop_p: float = 0.0):
+        """The level loop of cross_update_Y on fused projections, without autograd: the three
+        projections of the span nodes are one GEMM, the key/value projections of each level's
+        children another, and each level's kernel reads its operands as column slices of those
+        results.  Every level writes twice: a dense [B, P, D] block that feeds the next level's
+        GEMM, and its slice of the level-concatenated [B, N-1, D] result (returned, before
+        out_proj_y).  Unless `keep`, the last levels (few rows each) run as one launch that does
+        their projections on chip.  `keep` returns what a backward pass needs as a dict; `drop_p`
+        is the dropout probability applied to the children's values (the reference applies it
+        twice to the leaves' values)."""
         B, N, D = x.shape
         H, Dh = self.num_heads, self.head_dim
         _lib.require_gpu(x, y_in)
         cdt = self._compute_dtype(x)
         x, y_in = x.to(cdt).contiguous(), y_in.to(cdt).contiguous()
-        qkv = F.linear(y_in, self._fused_weight("qkv_y", (self.Wq_y, self.Wk_y, self.Wv_y), cdt))  # [B, N-1, 3D]
+        w_qkv = self._fused_weight("qkv_y", (self.Wq_y, self.Wk_y, self.Wv_y), cdt)
+        qkv = F.linear(y_in, w_qkv)  # [B, N-1, 3D]
         w_kv = self._fused_weight("kv_y", (self.Wk_y, self.Wv_y), cdt)
         # every buffer the kernels address by raw pointer has the one element type
         assert qkv.dtype == cdt and qkv.is_contiguous(), "projection result has an unexpected layout"
@@ -144,10 +172,11 @@ class HierarchicalAttention(nn.Module):
         fwd, code, stream = _lib.lib().hsa_build_parents_strided_fwd, _lib.dtype_code(x), _lib.stream_of(x)
         qkv_p, blk_p, out_p = qkv.data_ptr(), blocks.data_ptr(), y_new.data_ptr()
         # child rows the fused upper levels take (0: shape not handled)
-        top_rows = _lib.lib().hsa_cross_update_top_rows(H, Dh, code) if self.fuse_top_levels else 0
+        top_rows = 0 if keep or not self.fuse_top_levels else _lib.lib().hsa_cross_update_top_rows(H, Dh, code)
+        kvs, masks = [], []
         src, off = x, 0
         with torch.cuda.device(x.device):
-            for P in self.sizes:
+            for lvl, P in enumerate(self.sizes):
                 if 2 * P <= top_rows:
                     # the remaining levels fit one workgroup per batch: a single launch
                     w_top = self._fused_weight("kv_y_packed", (self.Wk_y, self.Wv_y), cdt, packed=True)
@@ -159,15 +188,73 @@ class HierarchicalAttention(nn.Module):
                     break
                 kv = F.linear(src, w_kv)  # [B, 2P, 2D]
                 assert kv.dtype == cdt and kv.is_contiguous(), "projection result has an unexpected layout"
+                if drop_p > 0:
+                    # dropout on the value half, as a saved multiplicative mask
+                    keep_p = 1.0 - drop_p
+                    m = torch.bernoulli(torch.full((B, 2 * P, D), keep_p, dtype=cdt, device=x.device)).div_(keep_p)
+                    if lvl == 0:
+                        m.mul_(torch.bernoulli(torch.full_like(m, keep_p)).div_(keep_p))
+                    kv[:, :, D:].mul_(m)
+                    masks.append(m)
                 par, kv_p, lvl_p = qkv_p + off * 3 * D * es, kv.data_ptr(), blk_p + B * off * D * es
                 rc = fwd(par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es, lvl_p,
                          out_p + off * D * es, B, P, H, Dh,
                          A((N - 1) * 3 * D, (N - 1) * 3 * D, (N - 1) * 3 * D, 4 * P * D, 4 * P * D, P * D,
                            (N - 1) * D), row_strides, code, stream)
                 _lib.check(rc, "hsa_build_parents_strided_fwd")
+                if keep:
+                    kvs.append(kv)
                 src = blocks[B * off * D:B * (off + P) * D].view(B, P, D)
                 off += P
-        return self.out_proj_y(y_new)
+        if not keep:
+            return y_new
+        return y_new, {"x": x, "y_in": y_in, "qkv": qkv, "blocks": blocks, "kvs": kvs, "masks": masks,
+                       "w_qkv": w_qkv, "w_kv": w_kv}
+
+    def _span_levels_backward(self, dy: torch.Tensor, kept: dict):
+        """Gradients of `_span_levels` with respect to x, y_in and the stacked q|k|v weights:
+        per level one kernel (the three weights are recomputed, every gradient row written once
+        into the fused layouts) and two GEMMs (input gradient and weight gradient of the fused
+        key/value projection).  Returns (dx, dy_in, dW_qkv [3D, D] fp32)."""
+        x, y_in, qkv, blocks = kept["x"], kept["y_in"], kept["qkv"], kept["blocks"]
+        kvs, masks, w_qkv, w_kv = kept["kvs"], kept["masks"], kept["w_qkv"], kept["w_kv"]
+        B, N, D = x.shape
+        H, Dh = self.num_heads, self.head_dim
+        cdt, es = x.dtype, x.element_size()
+        dy = dy.to(cdt).contiguous()
+        dqkv = torch.empty_like(qkv)
+        dw_kv = torch.zeros((2 * D, D), dtype=torch.float32, device=x.device)
+        A = ctypes.c_int64 * 11
+        bwd, code, stream = _lib.lib().hsa_build_parents_strided_bwd, _lib.dtype_code(x), _lib.stream_of(x)
+        rs = A(D, 3 * D, 3 * D, 3 * D, 2 * D, 2 * D, 3 * D, 3 * D, 3 * D, 2 * D, 2 * D)
+        T3 = (N - 1) * 3 * D
+        d_above, dx = None, None
+        with torch.cuda.device(x.device):
+            for lvl in range(len(self.sizes) - 1, -1, -1):
+                P, off = self.sizes[lvl], self.offsets[lvl]
+                g = dy[:, off:off + P]
+                g = (g + d_above) if d_above is not None else g.contiguous()
+                kv = kvs[lvl]
+                dkv = torch.empty_like(kv)
+                par, dpar = qkv.data_ptr() + off * 3 * D * es, dqkv.data_ptr() + off * 3 * D * es
+                kv_p, dkv_p = kv.data_ptr(), dkv.data_ptr()
+                rc = bwd(g.data_ptr(), par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es,
+                         dpar, dpar + D * es, dpar + 2 * D * es, dkv_p, dkv_p + D * es, B, P, H, Dh,
+                         A(P * D, T3, T3, T3, 4 * P * D, 4 * P * D, T3, T3, T3, 4 * P * D, 4 * P * D), rs, code, stream)
+                _lib.check(rc, "hsa_build_parents_strided_bwd")
+                if masks:
+                    dkv[:, :, D:].mul_(masks[lvl])
+                src = x if lvl == 0 else blocks[B * self.offsets[lvl - 1] * D:B * off * D].view(B, 2 * P, D)
+                dw_kv += torch.matmul(dkv.reshape(-1, 2 * D).t(), src.reshape(-1, D)).float()
+                d_src = torch.matmul(dkv, w_kv)  # [B, 2P, D]
+                if lvl == 0:
+                    dx = d_src
+                else:
+                    d_above = d_src
+        dy_in = torch.matmul(dqkv, w_qkv)
+        dw_qkv = torch.matmul(dqkv.reshape(-1, 3 * D).t(), y_in.reshape(-1, D)).float()
+        dw_qkv[D:] += dw_kv
+        return dx, dy_in, dw_qkv
 
     # -- bottom-up: leaves -> span nodes ----------------------------------------
     def cross_update_Y(self, x: torch.Tensor, y_in: torch.Tensor) -> torch.Tensor:
@@ -179,8 +266,13 @@ class HierarchicalAttention(nn.Module):
             self.sizes, self.offsets = self._build_level_info(N)
 
         grad = self._needs_autograd((x, y_in), (self.Wq_y, self.Wk_y, self.Wv_y))
-        if not grad and not (self.training and self.dropout.p > 0):
-            return self._cross_update_Y_direct(x, y_in)
+        drop_p = self.dropout.p if self.training else 0.0
+        if not grad and drop_p == 0:
+            return self.out_proj_y(self._span_levels(x, y_in))
+        if self.fused_training and x.is_cuda and N >= 2:
+            # the same fused level loop as one differentiable function
+            y_new = _SpanLevels.apply(self, drop_p, x, y_in, self.Wq_y.weight, self.Wk_y.weight, self.Wv_y.weight)
+            return self.out_proj_y(y_new)
 
         q_lv = torch.split(self._heads(self.Wq_y(y_in)), self.sizes, dim=1)
         k_lv = torch.split(self._heads(self.Wk_y(y_in)), self.sizes, dim=1)

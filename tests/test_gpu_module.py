@@ -84,10 +84,11 @@ def test_reference_check_configuration_cross_update_y():
     """The configuration of the reference's cross_update_Y check
     (hierarchical_attention_project/Hierarchical_Attention_Triton_Test.py:419-490): B=2, N=32768,
     16 heads of 64 (dim 1024), fp16, default nn.Linear init, inputs randn.clamp(-1, 1), eval mode,
-    dropout 0; its bar is 1e-2 max-abs on the output, used here as well.  Both paths of the module
-    are checked: the no-autograd one (fused projections, fused upper levels) and the forward of
-    the differentiable level-by-level one the reference's check runs.  The oracle is evaluated in
-    fp32 on the CPU (fp64 would take minutes at this size)."""
+    dropout 0; its bar is 1e-2 max-abs on the output, used here as well.  All three paths of the
+    module are checked: the no-autograd one (fused projections, fused upper levels) and the
+    forward of the two differentiable ones (fused level loop as one function; one projection and
+    one op per level as in the reference).  The oracle is evaluated in fp32 on the CPU (fp64
+    would take minutes at this size)."""
     B, N, H, Dh = 2, 32768, 16, 64
     dim = H * Dh
     torch.manual_seed(0)
@@ -99,9 +100,11 @@ def test_reference_check_configuration_cross_update_y():
     want = oracle.cross_update_y_ref(x.float(), y.float(), w, H)
     with torch.no_grad():
         fused = m.cross_update_Y(x.to(DEV), y.to(DEV))
+    fused_fn = m.cross_update_Y(x.to(DEV).requires_grad_(True), y.to(DEV).requires_grad_(True))
+    m.fused_training = False
     stepwise = m.cross_update_Y(x.to(DEV).requires_grad_(True), y.to(DEV).requires_grad_(True))
-    assert stepwise.requires_grad
-    for name, got in (("fused", fused), ("level by level", stepwise)):
+    assert stepwise.requires_grad and fused_fn.requires_grad
+    for name, got in (("fused", fused), ("fused, differentiable", fused_fn), ("level by level", stepwise)):
         err = float((got.detach().float().cpu() - want).abs().max())
         assert err < 1e-2, "%s: max abs err %.3e" % (name, err)
 
@@ -261,6 +264,95 @@ def test_fused_weight_cache_follows_weight_updates():
     a4, b4 = both()
     assert (a4.float() - b4.float()).abs().max() < 3e-2
     assert (a4.float() - a3.float()).abs().max() > 1e-3
+
+
+# ---------------------------------------------------------------- differentiable fused span-node update
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 64, 64, 2), (1, 256, 128, 4), (2, 2, 32, 1), (1, 1024, 512, 8)])
+def test_fused_span_node_update_gradients(dtype, shape):
+    """cross_update_Y with autograd runs the fused level loop as one differentiable function:
+    gradients with respect to the leaves, the span nodes and the three projection weights against
+    autograd through the fp64 oracle, and against the level-by-level path of the module."""
+    B, N, dim, H = shape
+    torch.manual_seed(20)
+    m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=4).to(DEV).to(dtype)
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(B, N, dim, generator=g).clamp(-1, 1).to(dtype)
+    y = torch.randn(B, N - 1, dim, generator=g).clamp(-1, 1).to(dtype)
+    dout = torch.randn(B, N - 1, dim, generator=g).to(dtype)
+    w = {k: v.detach().double().cpu().requires_grad_(True) for k, v in m.state_dict().items()}
+    xr, yr = x.double().requires_grad_(True), y.double().requires_grad_(True)
+    oracle.cross_update_y_ref(xr, yr, w, H).backward(dout.double())
+
+    def run(fused):
+        m.fused_training = fused
+        m.zero_grad()
+        xd, yd = x.to(DEV).requires_grad_(True), y.to(DEV).requires_grad_(True)
+        out = m.cross_update_Y(xd, yd)
+        out.backward(dout.to(DEV))
+        return out.detach(), xd.grad, yd.grad, {n: p.grad.clone() for n, p in m.named_parameters() if p.grad is not None}
+
+    out_f, dx_f, dy_f, dw_f = run(True)
+    out_s, dx_s, dy_s, dw_s = run(False)
+    assert set(dw_f) == set(dw_s) == {"Wq_y.weight", "Wk_y.weight", "Wv_y.weight", "out_proj_y.weight", "out_proj_y.bias"}
+    tol = 2e-4 if dtype == torch.float32 else 4e-2
+
+    def close(got, ref, what):
+        err = float((got.double().cpu() - ref).abs().max())
+        assert err <= tol * max(1.0, float(ref.abs().max())), "%s: max abs err %.3e (scale %.2f)" % (
+            what, err, float(ref.abs().max()))
+
+    close(out_f, oracle.cross_update_y_ref(xr, yr, w, H).detach(), "output")
+    close(dx_f, xr.grad, "dX")
+    close(dy_f, yr.grad, "dY")
+    for n in dw_f:
+        close(dw_f[n], w[n].grad, "d" + n)
+        close(dw_f[n], dw_s[n].double().cpu(), "d%s vs level-by-level path" % n)
+    close(dx_f, dx_s.double().cpu(), "dX vs level-by-level path")
+
+
+def test_fused_span_node_update_with_dropout():
+    """Training mode with dropout: the fused function draws its own masks for the children's
+    values (twice for the leaves', like the reference); forward and gradients must equal an
+    explicit composition of the oracle op with those same masks."""
+    B, N, dim, H, p = 2, 32, 64, 2, 0.25
+    torch.manual_seed(22)
+    m = sa.HierarchicalAttention(dim, H, dropout=p, window_size=4).to(DEV).train()
+    x = torch.randn(B, N, dim, device=DEV).requires_grad_(True)
+    y = torch.randn(B, N - 1, dim, device=DEV).requires_grad_(True)
+    m.sizes, m.offsets = m._build_level_info(N)
+    with torch.no_grad():
+        y_plain, _ = m._span_levels(x.detach(), y.detach(), keep=True, drop_p=0.0)
+    y_new, kept = m._span_levels(x.detach(), y.detach(), keep=True, drop_p=p)
+    assert (y_new - y_plain).abs().max() > 1e-3
+    masks = [mk.double().cpu() for mk in kept["masks"]]
+    assert len(masks) == len(m.sizes) and all(((mk == 0) | (mk > 1)).all() for mk in masks)
+    frac0 = float((masks[0] == 0).double().mean())
+    assert abs(frac0 - (1 - (1 - p) ** 2)) < 0.05          # two rounds of dropout on the leaves' values
+    # the same computation in fp64 with the masks put in by hand
+    w = {k: v.detach().double().cpu() for k, v in m.state_dict().items()}
+    xr, yr = x.detach().double().cpu().requires_grad_(True), y.detach().double().cpu().requires_grad_(True)
+    Dh = dim // H
+    lin = torch.nn.functional.linear
+    qp, kp, vp = (lin(yr, w[n]).view(B, -1, H, Dh) for n in ("Wq_y.weight", "Wk_y.weight", "Wv_y.weight"))
+    src, off, outs = xr, 0, []
+    for lvl, P in enumerate(m.sizes):
+        kc = lin(src, w["Wk_y.weight"]).view(B, -1, H, Dh)
+        vc = (lin(src, w["Wv_y.weight"]) * masks[lvl]).view(B, -1, H, Dh)
+        src = oracle.build_parent_nodes_ref(qp[:, off:off + P], kp[:, off:off + P], vp[:, off:off + P], kc, vc).reshape(B, P, dim)
+        outs.append(src)
+        off += P
+    want = torch.cat(outs, 1)
+    assert (y_new.double().cpu() - want).abs().max() < 1e-4
+    dout = torch.randn(B, N - 1, dim, dtype=torch.float64)
+    want.backward(dout)
+    dx, dy_in, dw = m._span_levels_backward(dout.to(DEV).float(), kept)
+    assert (dx.double().cpu() - xr.grad).abs().max() < 1e-4 * max(1.0, float(xr.grad.abs().max()))
+    assert (dy_in.double().cpu() - yr.grad).abs().max() < 1e-4 * max(1.0, float(yr.grad.abs().max()))
+    # and through the public method: gradients arrive at every trainable tensor
+    out = m.cross_update_Y(x, y)
+    out.square().mean().backward()
+    assert x.grad is not None and y.grad is not None and m.Wv_y.weight.grad is not None
 
 
 # ---------------------------------------------------------------- the reference's import name
