@@ -39,6 +39,13 @@ struct BwdTileParams {
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 
+// Query blocks (key blocks) one wavefront of the backward passes walks: 4 where the operands that
+// slide along the strip (leaf blocks in the query pass, query blocks in the key pass: NBW+1 when
+// causal, 2 NBW+1 otherwise) fit the registers, else 1.
+constexpr int bwd_strip_blocks(int D, int nbw, bool causal) {
+    return ((causal ? nbw + 1 : 2 * nbw + 1) <= 3 && D <= 64) ? 4 : 1;
+}
+
 template <typename T, int D>
 struct BwdTile {
     using M_ = Mma<T>;
@@ -104,7 +111,15 @@ struct BwdTile {
 // ---------------------------------------------------------------------------------------------
 // (A) query-stationary pass
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int NBW, bool CAUSAL>
+// A wavefront walks a strip of SB consecutive query blocks (SB * 16 <= 64 queries, aligned): the
+// leaf key / value operands slide along the strip in registers (each leaf row is fetched once per
+// strip), the far tree block (levels >= 6, the same nodes for the whole strip) is fetched once,
+// and the partial rows it collects are summed over the strip's blocks before they are written.
+// The next block's rows are requested while the current block is computed.
+//
+// Partial rows (fp32): levels 4 and 5 per query block, [2][B][N/16][H][2][D] (dK then dV);
+// levels >= 6 per strip, [2][B][N/16/SB][H][L-6][D], right behind.
+template <typename T, int D, int NBW, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(BWD_WPB * 64)
 attn_bwd_tile_query_kernel(BwdTileParams p) {
     using BT = BwdTile<T, D>;
@@ -123,31 +138,35 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
 
     const int N = p.N, L = p.L, R = p.R, H = p.H;
-    const int NB = N / TILE_Q;
+    const int NB = N / TILE_Q, NS = NB / SB;
     const int h = unit % H;
-    const int blk = (unit / H) % NB;
-    const int b = unit / (H * NB);
-    const int q0 = blk * TILE_Q;
+    const int strip = (unit / H) % NS;
+    const int b = unit / (H * NS);
+    const int blk0 = strip * SB;
+    const int qs = blk0 * TILE_Q;  // first query of the strip
     const size_t rs = (size_t)H * D;
     const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
     const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
     const uint16_t *Kb = p.k + ((size_t)b * p.M * H + h) * D + 8 * lchk;
     const uint16_t *Vb = p.v + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
 
     // ---- tree slot constants (same slot layout as the forward kernel) -------------------------
-    int t_row[NLD], u_row[NLD];     // rows this lane fetches / stores, -1 = slot does not exist
+    int t_lvl[NLD], t_add[NLD], t_xor[NLD], u_row[NLD];  // rows this lane fetches; u_row -1 = no such slot
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int sl = i * RPI + lrow;
-        int lvl, add, x;
-        if (sl < 8) { lvl = 1; add = sl; x = 0; }
-        else if (sl < 12) { lvl = 2; add = sl - 8; x = 0; }
-        else if (sl < 14) { lvl = 3; add = sl - 12; x = 0; }
-        else { lvl = 4 + (sl - 14); add = 0; x = 1; }
-        t_row[i] = lvl < L ? level_offset(N, lvl) + (((q0 >> lvl) + add) ^ x) : -1;
+        if (sl < 8) { t_lvl[i] = 1; t_add[i] = sl; t_xor[i] = 0; }
+        else if (sl < 12) { t_lvl[i] = 2; t_add[i] = sl - 8; t_xor[i] = 0; }
+        else if (sl < 14) { t_lvl[i] = 3; t_add[i] = sl - 12; t_xor[i] = 0; }
+        else { t_lvl[i] = 4 + (sl - 14); t_add[i] = 0; t_xor[i] = 1; }
         const int ul = 6 + sl;
-        u_row[i] = ul < L ? level_offset(N, ul) + ((q0 >> ul) ^ 1) : -1;
+        u_row[i] = ul < L ? level_offset(N, ul) + ((qs >> ul) ^ 1) : -1;
     }
+    auto near_row = [&](int i, int q0) {  // -1 = the slot's level does not exist
+        return t_lvl[i] < L ? level_offset(N, t_lvl[i]) + (((q0 >> t_lvl[i]) + t_add[i]) ^ t_xor[i]) : -1;
+    };
     auto slot_level = [](int sl, int &pl) {  // near slot -> level, position under the ancestor (-1: sibling slot)
         if (sl < 8) { pl = sl; return 1; }
         if (sl < 12) { pl = sl - 8; return 2; }
@@ -155,46 +174,15 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
         pl = -1;
         return 4 + (sl - 14);
     };
-    // orientation 1 (lane = query r16, regs = slots 4g+i) and orientation 2 (lane = slot r16,
-    // regs = queries 4g+i) liveness of the near and far blocks
-    float b1T[4], b1U[4], b2T[4], b2U[4];
+    // far block liveness in orientation 1 (lane = query r16, regs = slots 4g+i) and orientation 2
+    // (lane = slot r16, regs = queries 4g+i): the same for every block of the strip
+    float b1U[4], b2U[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        {
-            int pl;
-            const int lvl = slot_level(4 * g + i, pl);
-            bool live = pl >= 0 ? (pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1)))
-                                : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
-            b1T[i] = live ? 0.f : NEG_INF;
-            const int ul = 6 + 4 * g + i;
-            b1U[i] = (ul < L && (!CAUSAL || ((q0 >> ul) & 1))) ? 0.f : NEG_INF;
-        }
-        {
-            int pl;
-            const int lvl = slot_level(r16, pl);
-            const int ql = 4 * g + i;
-            bool live = pl >= 0 ? (pl == ((ql >> lvl) ^ 1) && (!CAUSAL || ((ql >> lvl) & 1)))
-                                : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
-            b2T[i] = live ? 0.f : NEG_INF;
-            const int ul = 6 + r16;
-            b2U[i] = (ul < L && (!CAUSAL || ((q0 >> ul) & 1))) ? 0.f : NEG_INF;
-        }
-    }
-    float biasL[NKL][4];
-#pragma unroll
-    for (int c = 0; c < NKL; ++c) {
-        const int dlt = TILE_Q * (c - NBW);
-        const int kb = blk - NBW + c;
-        const bool inside = kb >= 0 && kb < NB;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int kl = 4 * g + i;
-            const int diff = dlt + kl - r16;
-            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
-            const bool sib = dlt == 0 && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
-            const int cnt = (int)win + (int)sib;
-            biasL[c][i] = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
-        }
+        const int ul1 = 6 + 4 * g + i;
+        b1U[i] = (ul1 < L && (!CAUSAL || ((qs >> ul1) & 1))) ? 0.f : NEG_INF;
+        const int ul2 = 6 + r16;
+        b2U[i] = (ul2 < L && (!CAUSAL || ((qs >> ul2) & 1))) ? 0.f : NEG_INF;
     }
 
     // ---- loads ------------------------------------------------------------------------------
@@ -203,176 +191,285 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) dst[i] = *reinterpret_cast<const u32x4_t *>(ptr + (size_t)(i * RPI) * rs);
     };
-    auto load_rows = [&](const uint16_t *base, const int (&rows)[NLD], u32x4_t (&dst)[NLD]) {
-#pragma unroll
-        for (int i = 0; i < NLD; ++i)
-            dst[i] = *reinterpret_cast<const u32x4_t *>(base + (size_t)(rows[i] < 0 ? q0 : rows[i]) * rs);
+    auto leaf_row0 = [&](int kb) {
+        kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
+        return kb * TILE_Q;
     };
-    // ---- loads and operand forms (each block: rows -> LDS -> MFMA pieces) -----------------------
-    u32x4_t Qf[KS], Gf[KS], Kc[NKB][KS], Vc[NKB][KS];
+    struct Stage {
+        u32x4_t q[NLD], g[NLD], k[NLD], v[NLD], kt[NLD], vt[NLD];
+    };
+    auto request = [&](Stage &sg, int blk) {
+        const int q0 = blk * TILE_Q;
+        load_block(Qb, q0, sg.q);
+        load_block(Gb, q0, sg.g);
+        const int row0 = leaf_row0(blk - NBW + NKL - 1);  // the leaf block that enters with this query block
+        load_block(Kb, row0, sg.k);
+        load_block(Vb, row0, sg.v);
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int tr = near_row(i, q0);
+            sg.kt[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(tr < 0 ? q0 : tr) * rs);
+            sg.vt[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(tr < 0 ? q0 : tr) * rs);
+        }
+    };
+
+    // everything the first block needs is requested before anything is consumed
+    u32x4_t Kc[NKB][KS], Vc[NKB][KS];
+    Stage st[SB];
     {
-        u32x4_t rQ[NLD], rG[NLD];
-        load_block(Qb, q0, rQ);
-        load_block(Gb, q0, rG);
-        bt.put(0, rQ);
-        bt.put(1, rG);
+        u32x4_t rKu[NLD], rVu[NLD], rKh[NKL][NLD], rVh[NKL][NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            rKu[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
+            rVu[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
+        }
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+            load_block(Kb, leaf_row0(blk0 - NBW + c), rKh[c]);
+            load_block(Vb, leaf_row0(blk0 - NBW + c), rVh[c]);
+        }
+        request(st[0], blk0);
+        bt.put(2, rKu);
+        bt.put(3, rVu);
+        bt.get(2, Kc[NKL + 1]);
+        bt.get(3, Vc[NKL + 1]);
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+            bt.put(2, rKh[c]);
+            bt.put(3, rVh[c]);
+            bt.get(2, Kc[c]);
+            bt.get(3, Vc[c]);
+        }
+    }
+    // partial rows of the far block, summed over the strip
+    f32x4 fk[NJ], fv[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+#pragma unroll
+    for (int it = 0; it < SB; ++it) {
+        const int blk = blk0 + it;
+        const int q0 = blk * TILE_Q;
+        Stage &sg = st[it];
+        // rows -> operand pieces; then the next block's rows are requested
+        u32x4_t Qf[KS], Gf[KS];
+        bt.put(0, sg.q);
+        bt.put(1, sg.g);
+        bt.put(2, sg.k);
+        bt.put(3, sg.v);
         bt.get(0, Qf);
         bt.get(1, Gf);
-    }
-#pragma unroll
-    for (int c = 0; c < NKB; ++c) {
-        u32x4_t rK[NLD], rV[NLD];
-        if (c < NKL) {
-            int kb = blk - NBW + c;
-            kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
-            load_block(Kb, kb * TILE_Q, rK);
-            load_block(Vb, kb * TILE_Q, rV);
-        } else if (c == NKL) {
-            load_rows(Kb, t_row, rK);
-            load_rows(Vb, t_row, rV);
-        } else {
-            load_rows(Kb, u_row, rK);
-            load_rows(Vb, u_row, rV);
-        }
-        bt.put(2, rK);
-        bt.put(3, rV);
-        bt.get(2, Kc[c]);
-        bt.get(3, Vc[c]);
-    }
+        bt.get(2, Kc[NKL - 1]);
+        bt.get(3, Vc[NKL - 1]);
+        bt.put(2, sg.kt);
+        bt.put(3, sg.vt);
+        bt.get(2, Kc[NKL]);
+        bt.get(3, Vc[NKL]);
+        if (it + 1 < SB) request(st[it + 1 < SB ? it + 1 : it], blk + 1);
 
-    // ---- orientation 1: S^T, dP^T [key, query] ---------------------------------------------------
-    float sc[NKB][4], dp[NKB][4];
-    float mx = NEG_INF;
+        // liveness of the near block and of the leaf blocks for this query block
+        int t_row[NLD];
 #pragma unroll
-    for (int c = 0; c < NKB; ++c) {
-        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            a = M_::k32(Kc[c][ks], Qf[ks], a);
-            d = M_::k32(Vc[c][ks], Gf[ks], d);
-        }
+        for (int i = 0; i < NLD; ++i) t_row[i] = near_row(i, q0);
+        float b1T[4], b2T[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
-            sc[c][i] = fmaf(a[i], p.scale_log2e, bias);
-            dp[c][i] = d[i];
-            mx = fmaxf(mx, sc[c][i]);
+            {
+                int pl;
+                const int lvl = slot_level(4 * g + i, pl);
+                const bool live = pl >= 0 ? (pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1)))
+                                          : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+                b1T[i] = live ? 0.f : NEG_INF;
+            }
+            {
+                int pl;
+                const int lvl = slot_level(r16, pl);
+                const int ql = 4 * g + i;
+                const bool live = pl >= 0 ? (pl == ((ql >> lvl) ^ 1) && (!CAUSAL || ((ql >> lvl) & 1)))
+                                          : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+                b2T[i] = live ? 0.f : NEG_INF;
+            }
         }
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    float den = 0.f;
+        float biasL[NKL][4];
 #pragma unroll
-    for (int c = 0; c < NKB; ++c)
+        for (int c = 0; c < NKL; ++c) {
+            const int dlt = TILE_Q * (c - NBW);
+            const int kb = blk - NBW + c;
+            const bool inside = kb >= 0 && kb < NB;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sc[c][i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
-            den += sc[c][i];
+            for (int i = 0; i < 4; ++i) {
+                const int kl = 4 * g + i;
+                const int diff = dlt + kl - r16;
+                const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+                const bool sib = dlt == 0 && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
+                const int cnt = (int)win + (int)sib;
+                biasL[c][i] = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+            }
         }
-    den += __shfl_xor(den, 16, 64);
-    den += __shfl_xor(den, 32, 64);
-    const float inv = 1.0f / den;
-    float delta = 0.f;
-#pragma unroll
-    for (int c = 0; c < NKB; ++c)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sc[c][i] *= inv;  // P
-            delta = fmaf(sc[c][i], dp[c][i], delta);
-        }
-    delta += __shfl_xor(delta, 16, 64);
-    delta += __shfl_xor(delta, 32, 64);
-    const float lse = mx + __builtin_amdgcn_logf(den);  // log2 domain: P = exp2(s' - lse)
-    if (g == 0) {
-        float *st = p.stats + (((size_t)b * N + q0 + r16) * H + h) * 2;
-        st[0] = lse;
-        st[1] = delta;
-    }
 
-    // ---- dQ^T = sum_c K_c^T . dS_c^T ---------------------------------------------------------------
-    {
-        f32x4 acc[NJ];
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // ---- orientation 1: S^T, dP^T [key, query] ---------------------------------------------------
+        float sc[NKB][4], dp[NKB][4];
+        float mx = NEG_INF;
 #pragma unroll
         for (int c = 0; c < NKB; ++c) {
-            u32x2_t KT[NJ];
-            bt.transpose(Kc[c], KT);
-            float ds[4];
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ds[i] = sc[c][i] * (dp[c][i] - delta) * p.scale;
-            const u32x2_t dsp = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+            for (int ks = 0; ks < KS; ++ks) {
+                a = M_::k32(Kc[c][ks], Qf[ks], a);
+                d = M_::k32(Vc[c][ks], Gf[ks], d);
+            }
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) acc[j] = M_::k16(KT[j], dsp, acc[j]);
+            for (int i = 0; i < 4; ++i) {
+                const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
+                sc[c][i] = fmaf(a[i], p.scale_log2e, bias);
+                dp[c][i] = d[i];
+                mx = fmaxf(mx, sc[c][i]);
+            }
         }
-        bt.put_result(0, acc, 1.0f);
-        uint16_t *optr = p.dq + ((size_t)b * N * H + h) * D + 8 * lchk + (size_t)(q0 + lrow) * rs;
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float den = 0.f;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i)
-            *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
-    }
+        for (int c = 0; c < NKB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[c][i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
+                den += sc[c][i];
+            }
+        den += __shfl_xor(den, 16, 64);
+        den += __shfl_xor(den, 32, 64);
+        const float inv = 1.0f / den;
+        float delta = 0.f;
+#pragma unroll
+        for (int c = 0; c < NKB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[c][i] *= inv;  // P
+                delta = fmaf(sc[c][i], dp[c][i], delta);
+            }
+        delta += __shfl_xor(delta, 16, 64);
+        delta += __shfl_xor(delta, 32, 64);
+        const float lse = mx + __builtin_amdgcn_logf(den);  // log2 domain: P = exp2(s' - lse)
+        if (g == 0) {
+            float *stp = p.stats + (((size_t)b * N + q0 + r16) * H + h) * 2;
+            stp[0] = lse;
+            stp[1] = delta;
+        }
 
-    // ---- orientation 2 for the tree blocks: dK^T, dV^T [channel, slot] ------------------------------
-    u32x2_t QT[NJ], GT[NJ];
-    bt.transpose(Qf, QT);
-    bt.transpose(Gf, GT);
-    float lse4[4], del4[4];
+        // ---- dQ^T = sum_c K_c^T . dS_c^T ---------------------------------------------------------------
+        {
+            f32x4 acc[NJ];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        lse4[i] = __shfl(lse, 4 * g + i, 64);
-        del4[i] = __shfl(delta, 4 * g + i, 64);
-    }
-    uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
-    uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+            for (int j = 0; j < NJ; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-        const int c = NKL + t;
-        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < NKB; ++c) {
+                u32x2_t KT[NJ];
+                bt.transpose(Kc[c], KT);
+                float ds[4];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            a = M_::k32(Qf[ks], Kc[c][ks], a);   // S[query 4g+i, slot r16]
-            d = M_::k32(Gf[ks], Vc[c][ks], d);   // dP[query, slot]
+                for (int i = 0; i < 4; ++i) ds[i] = sc[c][i] * (dp[c][i] - delta) * p.scale;
+                const u32x2_t dsp = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[j] = M_::k16(KT[j], dsp, acc[j]);
+            }
+            bt.put_result(0, acc, 1.0f);
+            uint16_t *optr = p.dq + ((size_t)b * N * H + h) * D + 8 * lchk + (size_t)(q0 + lrow) * rs;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i)
+                *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
         }
-        float pp[4], ds[4];
+
+        // ---- orientation 2 for the tree blocks: dK^T, dV^T [channel, slot] ------------------------------
+        u32x2_t QT[NJ], GT[NJ];
+        bt.transpose(Qf, QT);
+        bt.transpose(Gf, GT);
+        float lse4[4], del4[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float bias = t == 0 ? b2T[i] : b2U[i];
-            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
-            ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
+            lse4[i] = __shfl(lse, 4 * g + i, 64);
+            del4[i] = __shfl(delta, 4 * g + i, 64);
         }
-        const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
-        const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
-        f32x4 tk[NJ], tv[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            tk[j] = M_::k16(QT[j], dk, z);
-            tv[j] = M_::k16(GT[j], pk, z);
-        }
-        if (t == 0) {
-            // slots 0..13 (levels 1..3) are complete: rows written directly
-            bt.put_result(0, tk, 1.0f);
-            bt.put_result(1, tv, 1.0f);
+        for (int t = 0; t < 2; ++t) {
+            const int c = NKL + t;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int i = 0; i < NLD; ++i) {
-                const int sl = i * RPI + lrow;
-                if (sl < 14 && t_row[i] >= 0) {
-                    *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
-                    *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
+            for (int ks = 0; ks < KS; ++ks) {
+                a = M_::k32(Qf[ks], Kc[c][ks], a);   // S[query 4g+i, slot r16]
+                d = M_::k32(Gf[ks], Vc[c][ks], d);   // dP[query, slot]
+            }
+            float pp[4], ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float bias = t == 0 ? b2T[i] : b2U[i];
+                pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
+                ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
+            }
+            const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+            const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+            if (t == 0) {
+                f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    tk[j] = M_::k16(QT[j], dk, z);
+                    tv[j] = M_::k16(GT[j], pk, z);
+                }
+                // slots 0..13 (levels 1..3) are complete: rows written directly
+                bt.put_result(0, tk, 1.0f);
+                bt.put_result(1, tv, 1.0f);
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int sl = i * RPI + lrow;
+                    if (sl < 14 && t_row[i] >= 0) {
+                        *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
+                        *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
+                    }
+                }
+                // levels 4 and 5 collect from one or two blocks: this block's partial rows
+                const int lvl = r16 >= 14 ? 4 + (r16 - 14) : -1;
+                if (lvl >= 4 && lvl < L) {
+                    const size_t po = ((((size_t)b * NB + blk) * H + h) * 2 + (lvl - 4)) * D;
+                    float *pkp = p.partial + po;
+                    float *pvp = p.partial + (size_t)p.B * NB * H * 2 * D + po;
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                        *reinterpret_cast<f32x4 *>(pkp + ch) = tk[j];
+                        *reinterpret_cast<f32x4 *>(pvp + ch) = tv[j];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    fk[j] = M_::k16(QT[j], dk, fk[j]);
+                    fv[j] = M_::k16(GT[j], pk, fv[j]);
                 }
             }
         }
-        // slots of levels >= 4 collect from several blocks: this block's partial rows
-        const int lvl = t == 0 ? (r16 >= 14 ? 4 + (r16 - 14) : -1) : 6 + r16;
-        if (lvl >= 4 && lvl < L) {
-            const size_t po = ((((size_t)b * NB + blk) * H + h) * (L - 4) + (lvl - 4)) * D;
-            float *pk = p.partial + po;
-            float *pv = p.partial + (size_t)p.B * NB * H * (L - 4) * D + po;
+
+        // slide the leaf window by one block
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) { Kc[c][ks] = Kc[c + 1][ks]; Vc[c][ks] = Vc[c + 1][ks]; }
+        }
+    }
+
+    // levels >= 6: the strip's partial rows
+    {
+        const int lvl = 6 + r16;
+        const int LF = L - 6;
+        if (lvl < L) {
+            float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
+            const size_t po = ((((size_t)b * NS + strip) * H + h) * LF + (lvl - 6)) * D;
+            float *pkp = far + po;
+            float *pvp = far + (size_t)p.B * NS * H * LF * D + po;
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
                 const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
-                *reinterpret_cast<f32x4 *>(pk + ch) = tk[j];
-                *reinterpret_cast<f32x4 *>(pv + ch) = tv[j];
+                *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
+                *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
             }
         }
     }
@@ -381,13 +478,17 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
 // ---------------------------------------------------------------------------------------------
 // (B) key-stationary pass over the leaf key blocks
 // ---------------------------------------------------------------------------------------------
-template <typename T, int D, int NBW, bool CAUSAL>
+// A wavefront walks SB consecutive key blocks; the query blocks whose window reaches a key block
+// (NQB of them) slide along in registers in operand form, so each query / dO row is fetched once
+// per strip instead of once per key block it touches.
+template <typename T, int D, int NBW, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(BWD_WPB * 64)
 attn_bwd_tile_key_kernel(BwdTileParams p) {
     using BT = BwdTile<T, D>;
     using M_ = Mma<T>;
     constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD;
     constexpr int NQB = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // query blocks that reach a key block
+    constexpr int QOFF = CAUSAL ? 0 : -NBW;              // first of them, relative to the key block
     constexpr int LDS_SLOTS = 4;
     __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
 
@@ -399,11 +500,11 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
     const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
 
     const int N = p.N, R = p.R, H = p.H;
-    const int NB = N / TILE_Q;
+    const int NB = N / TILE_Q, NS = NB / SB;
     const int h = unit % H;
-    const int kb = (unit / H) % NB;
-    const int b = unit / (H * NB);
-    const int k0 = kb * TILE_Q;
+    const int strip = (unit / H) % NS;
+    const int b = unit / (H * NS);
+    const int kb0 = strip * SB;
     const size_t rs = (size_t)H * D;
     const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
     const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
@@ -415,88 +516,135 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) dst[i] = *reinterpret_cast<const u32x4_t *>(ptr + (size_t)(i * RPI) * rs);
     };
-    u32x4_t rK[NLD], rV[NLD], rQ[NQB][NLD], rG[NQB][NLD];
-    load_block(Kb, k0, rK);
-    load_block(Vb, k0, rV);
-    float lse4[NQB][4], del4[NQB][4];
-#pragma unroll
-    for (int c = 0; c < NQB; ++c) {
-        int qb = kb + (CAUSAL ? c : c - NBW);
-        qb = qb < 0 ? 0 : (qb >= NB ? NB - 1 : qb);
-        load_block(Qb, qb * TILE_Q, rQ[c]);
-        load_block(Gb, qb * TILE_Q, rG[c]);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float *st = p.stats + (((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h) * 2;
-            lse4[c][i] = st[0];
-            del4[c][i] = st[1];
-        }
-    }
-    u32x4_t Kf[KS], Vf[KS];
-    bt.put(0, rK);
-    bt.put(1, rV);
-    bt.get(0, Kf);
-    bt.get(1, Vf);
-
-    f32x4 tk[NJ], tv[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-#pragma unroll
-    for (int c = 0; c < NQB; ++c) {
-        const int qb = kb + (CAUSAL ? c : c - NBW);
-        const bool inside = qb >= 0 && qb < NB;  // uniform
+    auto clampb = [&](int qb) { return qb < 0 ? 0 : (qb >= NB ? NB - 1 : qb); };
+    // a query block in the forms the key pass needs
+    struct QBlock {
         u32x4_t Qf[KS], Gf[KS];
-        bt.put(2, rQ[c]);
-        bt.put(3, rG[c]);
-        bt.get(2, Qf);
-        bt.get(3, Gf);
         u32x2_t QT[NJ], GT[NJ];
-        bt.transpose(Qf, QT);
-        bt.transpose(Gf, GT);
-        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            a = M_::k32(Qf[ks], Kf[ks], a);  // S[query 4g+i of block qb, key r16]
-            d = M_::k32(Gf[ks], Vf[ks], d);
-        }
-        float pp[4], ds[4];
+        float lse4[4], del4[4];
+    };
+    struct Stage {
+        u32x4_t k[NLD], v[NLD], q[NLD], g[NLD];
+        float lse4[4], del4[4];
+    };
+    auto request = [&](Stage &sg, int kb) {  // key block kb and the query block that enters with it
+        load_block(Kb, kb * TILE_Q, sg.k);
+        load_block(Vb, kb * TILE_Q, sg.v);
+        const int qb = clampb(kb + QOFF + NQB - 1);
+        load_block(Qb, qb * TILE_Q, sg.q);
+        load_block(Gb, qb * TILE_Q, sg.g);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int ql = 4 * g + i;
-            const int diff = (kb - qb) * TILE_Q + r16 - ql;  // key - query
-            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
-            const bool sib = qb == kb && r16 == (ql ^ 1) && (!CAUSAL || (ql & 1));
-            const int cnt = (int)win + (int)sib;
-            const float bias = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
-            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[c][i]);
-            ds[i] = pp[i] * (d[i] - del4[c][i]) * p.scale;
+            const float *stp = p.stats + (((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h) * 2;
+            sg.lse4[i] = stp[0];
+            sg.del4[i] = stp[1];
         }
-        const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
-        const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+    };
+    auto absorb = [&](QBlock &qq, const u32x4_t (&rq)[NLD], const u32x4_t (&rg)[NLD], const float (&l4)[4],
+                      const float (&d4)[4]) {
+        bt.put(2, rq);
+        bt.put(3, rg);
+        bt.get(2, qq.Qf);
+        bt.get(3, qq.Gf);
+        bt.transpose(qq.Qf, qq.QT);
+        bt.transpose(qq.Gf, qq.GT);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            tk[j] = M_::k16(QT[j], dk, tk[j]);
-            tv[j] = M_::k16(GT[j], pk, tv[j]);
+        for (int i = 0; i < 4; ++i) { qq.lse4[i] = l4[i]; qq.del4[i] = d4[i]; }
+    };
+
+    QBlock qblk[NQB];
+    Stage st[SB];
+    {
+        // the query blocks carried into the first key block, then the first stage
+        u32x4_t rq[NQB][NLD], rg[NQB][NLD];
+        float l4[NQB][4], d4[NQB][4];
+#pragma unroll
+        for (int c = 0; c + 1 < NQB; ++c) {
+            const int qb = clampb(kb0 + QOFF + c);
+            load_block(Qb, qb * TILE_Q, rq[c]);
+            load_block(Gb, qb * TILE_Q, rg[c]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float *stp = p.stats + (((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h) * 2;
+                l4[c][i] = stp[0];
+                d4[c][i] = stp[1];
+            }
         }
+        request(st[0], kb0);
+#pragma unroll
+        for (int c = 0; c + 1 < NQB; ++c) absorb(qblk[c], rq[c], rg[c], l4[c], d4[c]);
     }
-    bt.put_result(0, tk, 1.0f);
-    bt.put_result(1, tv, 1.0f);
-    uint16_t *dKp = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
-    uint16_t *dVp = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
+
 #pragma unroll
-    for (int i = 0; i < NLD; ++i) {
-        *reinterpret_cast<u32x4_t *>(dKp + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
-        *reinterpret_cast<u32x4_t *>(dVp + (size_t)(i * RPI) * rs) = bt.get_row_piece(1, i);
+    for (int it = 0; it < SB; ++it) {
+        const int kb = kb0 + it;
+        const int k0 = kb * TILE_Q;
+        Stage &sg = st[it];
+        u32x4_t Kf[KS], Vf[KS];
+        bt.put(0, sg.k);
+        bt.put(1, sg.v);
+        bt.get(0, Kf);
+        bt.get(1, Vf);
+        absorb(qblk[NQB - 1], sg.q, sg.g, sg.lse4, sg.del4);
+        if (it + 1 < SB) request(st[it + 1 < SB ? it + 1 : it], kb + 1);
+
+        f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+#pragma unroll
+        for (int c = 0; c < NQB; ++c) {
+            const int qb = kb + QOFF + c;
+            const bool inside = qb >= 0 && qb < NB;  // uniform
+            const QBlock &qq = qblk[c];
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                a = M_::k32(qq.Qf[ks], Kf[ks], a);  // S[query 4g+i of block qb, key r16]
+                d = M_::k32(qq.Gf[ks], Vf[ks], d);
+            }
+            float pp[4], ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ql = 4 * g + i;
+                const int diff = (kb - qb) * TILE_Q + r16 - ql;  // key - query
+                const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+                const bool sib = qb == kb && r16 == (ql ^ 1) && (!CAUSAL || (ql & 1));
+                const int cnt = (int)win + (int)sib;
+                const float bias = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+                pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - qq.lse4[i]);
+                ds[i] = pp[i] * (d[i] - qq.del4[i]) * p.scale;
+            }
+            const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+            const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                tk[j] = M_::k16(qq.QT[j], dk, tk[j]);
+                tv[j] = M_::k16(qq.GT[j], pk, tv[j]);
+            }
+        }
+        bt.put_result(0, tk, 1.0f);
+        bt.put_result(1, tv, 1.0f);
+        uint16_t *dKp = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
+        uint16_t *dVp = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk + (size_t)(k0 + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            *reinterpret_cast<u32x4_t *>(dKp + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
+            *reinterpret_cast<u32x4_t *>(dVp + (size_t)(i * RPI) * rs) = bt.get_row_piece(1, i);
+        }
+        // slide the query blocks by one
+#pragma unroll
+        for (int c = 0; c + 1 < NQB; ++c) qblk[c] = qblk[c + 1];
     }
 }
 
 // Rows of tree levels >= 4 (and anything above row 2N-2): node (l, p) sums the partial rows of the
-// 2^(l-4) query blocks under its sibling; nodes nobody attends (the root, right-hand nodes when
-// causal, rows past 2N-1) get zeros.  One thread per (batch, row, head, channel).
+// query blocks (levels 4, 5) or strips (levels >= 6) under its sibling; nodes nobody attends (the
+// root, right-hand nodes when causal, rows past 2N-1) get zeros.  One thread per (batch, row,
+// head, channel).  lg_sb = log2 of the blocks per strip of the query pass.
 template <typename T>
 __global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ dk,
                                             uint16_t *__restrict__ dv, int B, int N, int M, int H, int D, int L,
-                                            int causal, int first_row) {
+                                            int causal, int first_row, int lg_sb) {
     const size_t per_b = (size_t)(M - first_row) * H * D;
     const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= (size_t)B * per_b) return;
@@ -511,22 +659,34 @@ __global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, u
         while (row >= level_offset(N, lvl + 1)) ++lvl;
         const int pidx = row - level_offset(N, lvl);
         if (!causal || (pidx & 1) == 0) {
-            const int NB = N / TILE_Q;
-            const int nblk = 1 << (lvl - 4);
-            const int blk0 = (pidx ^ 1) << (lvl - 4);
-            const size_t stride = (size_t)H * (L - 4) * D;
-            const float *pk = partial + (((size_t)b * NB + blk0) * H + h) * (L - 4) * D + (size_t)(lvl - 4) * D + d;
-            const float *pv = pk + (size_t)B * NB * H * (L - 4) * D;
-            // eight independent loads in flight per round trip (the top nodes sum up to N/32 rows)
+            const int NB = N / TILE_Q, NS = NB >> lg_sb;
+            const int blk0 = (pidx ^ 1) << (lvl - 4);  // first query block under the sibling
+            const float *pk, *pv;
+            size_t stride;
+            int n;
+            if (lvl < 6) {
+                n = 1 << (lvl - 4);
+                stride = (size_t)H * 2 * D;
+                pk = partial + (((size_t)b * NB + blk0) * H + h) * 2 * D + (size_t)(lvl - 4) * D + d;
+                pv = pk + (size_t)B * NB * H * 2 * D;
+            } else {
+                const int LF = L - 6;
+                n = (1 << (lvl - 4)) >> lg_sb;
+                stride = (size_t)H * LF * D;
+                const float *far = partial + 2 * (size_t)B * NB * H * 2 * D;
+                pk = far + (((size_t)b * NS + (blk0 >> lg_sb)) * H + h) * LF * D + (size_t)(lvl - 6) * D + d;
+                pv = pk + (size_t)B * NS * H * LF * D;
+            }
+            // eight independent loads in flight per round trip
             int i = 0;
-            for (; i + 8 <= nblk; i += 8) {
+            for (; i + 8 <= n; i += 8) {
                 float a[8], c[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) { a[u] = pk[(size_t)(i + u) * stride]; c[u] = pv[(size_t)(i + u) * stride]; }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) { vk += a[u]; vv += c[u]; }
             }
-            for (; i < nblk; ++i) {
+            for (; i < n; ++i) {
                 vk += pk[(size_t)i * stride];
                 vv += pv[(size_t)i * stride];
             }

@@ -4,30 +4,43 @@
 
 namespace hsa {
 
-template <typename T, int D, int NBW, bool CAUSAL>
-static int bwd_tile_launch_one(const BwdTileParams &p, hipStream_t st) {
-    const int nwg = (p.n_units + BWD_WPB - 1) / BWD_WPB;
-    attn_bwd_tile_query_kernel<T, D, NBW, CAUSAL><<<nwg, BWD_WPB * 64, 0, st>>>(p);
+// p.n_units counts 16-query blocks; a wavefront takes SB of them (4 when the sequence has that
+// many blocks and the variant's operands fit the registers, else 1)
+template <typename T, int D, int NBW, bool CAUSAL, int SB>
+static int bwd_tile_launch_sb(const BwdTileParams &p, hipStream_t st) {
+    BwdTileParams q = p;
+    q.n_units = p.n_units / SB;
+    const int nwg = (q.n_units + BWD_WPB - 1) / BWD_WPB;
+    attn_bwd_tile_query_kernel<T, D, NBW, CAUSAL, SB><<<nwg, BWD_WPB * 64, 0, st>>>(q);
     int rc = check_launch("attn_bwd_tile_query_kernel");
     if (rc != HSA_OK) return rc;
-    attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL><<<nwg, BWD_WPB * 64, 0, st>>>(p);
+    attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL, SB><<<nwg, BWD_WPB * 64, 0, st>>>(q);
     return check_launch("attn_bwd_tile_key_kernel");
 }
 
+template <typename T, int D, int NBW, bool CAUSAL>
+static int bwd_tile_launch_one(const BwdTileParams &p, int sb, hipStream_t st) {
+    if constexpr (bwd_strip_blocks(D, NBW, CAUSAL) == 4) {
+        if (sb == 4) return bwd_tile_launch_sb<T, D, NBW, CAUSAL, 4>(p, st);
+    }
+    if (sb != 1) return fail(HSA_ERR_INVALID, "internal: strip length %d not built for this variant", sb);
+    return bwd_tile_launch_sb<T, D, NBW, CAUSAL, 1>(p, st);
+}
+
 template <typename T, int D>
-int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, hipStream_t st);
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb, hipStream_t st);
 
 #define HSA_BWD_TILE_INSTANTIATE(T, D)                                                         \
     template <>                                                                                \
-    int attn_bwd_tile_launch_td<T, D>(const BwdTileParams &p, int nbw, bool causal,            \
+    int attn_bwd_tile_launch_td<T, D>(const BwdTileParams &p, int nbw, bool causal, int sb,    \
                                       hipStream_t st) {                                        \
         switch (nbw * 2 + (causal ? 1 : 0)) {                                                  \
-            case 0: return bwd_tile_launch_one<T, D, 0, false>(p, st);                         \
-            case 1: return bwd_tile_launch_one<T, D, 0, true>(p, st);                          \
-            case 2: return bwd_tile_launch_one<T, D, 1, false>(p, st);                         \
-            case 3: return bwd_tile_launch_one<T, D, 1, true>(p, st);                          \
-            case 4: return bwd_tile_launch_one<T, D, 2, false>(p, st);                         \
-            case 5: return bwd_tile_launch_one<T, D, 2, true>(p, st);                          \
+            case 0: return bwd_tile_launch_one<T, D, 0, false>(p, sb, st);                     \
+            case 1: return bwd_tile_launch_one<T, D, 0, true>(p, sb, st);                      \
+            case 2: return bwd_tile_launch_one<T, D, 1, false>(p, sb, st);                     \
+            case 3: return bwd_tile_launch_one<T, D, 1, true>(p, sb, st);                      \
+            case 4: return bwd_tile_launch_one<T, D, 2, false>(p, sb, st);                     \
+            case 5: return bwd_tile_launch_one<T, D, 2, true>(p, sb, st);                      \
         }                                                                                      \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward");    \
     }

@@ -20,7 +20,7 @@
 namespace hsa {
 
 template <typename T, int D>
-int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, hipStream_t st);
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb, hipStream_t st);
 
 // ---------------------------------------------------------------- parent build
 template <typename T, int VEC> struct BPack { typename T::storage e[VEC]; };
@@ -648,8 +648,10 @@ static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype)
 static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
     return 2 * (size_t)B * N * H * (2 * R + 1 + L);
 }
+// statistics [B,N,H,2] + partial rows of dK and dV: levels 4 and 5 per query block, levels >= 6 per
+// strip (sized for strips of one block)
 static size_t bwd_tile_ws_floats(int B, int N, int H, int D, int L) {
-    const size_t lv = L > 4 ? L - 4 : 0;
+    const size_t lv = 2 + (L > 6 ? L - 6 : 0);
     return (size_t)B * N * H * 2 + 2 * (size_t)B * (N / TILE_Q) * H * lv * D;
 }
 
@@ -669,15 +671,17 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.scale = 1.0f / sqrtf((float)D);
     p.scale_log2e = 1.4426950408889634f * p.scale;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
-    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, st)
-           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, st)
-                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, st);
+    const int NB = N / TILE_Q;
+    const int sb = NB % 4 == 0 ? bwd_strip_blocks(D, nbw, causal != 0) : 1;
+    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, st)
+           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
+                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
     if (rc != HSA_OK) return rc;
     const int first = level_offset(N, 4);
     const size_t n_fin = (size_t)B * (M - first) * H * D;
     if (n_fin) {
         attn_bwd_tile_reduce_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
-            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first);
+            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, sb == 4 ? 2 : 0);
         rc = check_launch("attn_bwd_tile_reduce_kernel");
     }
     return rc;

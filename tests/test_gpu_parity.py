@@ -776,7 +776,8 @@ def _grad_close(got, want, dtype, what):
                                   (1, 32, 2, 20, 0, None), (1, 16, 2, 16, 20, 40), (1, 16, 2, 64, 3, None),
                                   (2, 256, 3, 64, 32, 600), (1, 1024, 2, 64, 0, None), (1, 64, 12, 64, 9, None),
                                   (1, 128, 2, 128, 32, None), (2, 32, 3, 128, 7, None), (2, 256, 4, 32, 16, None),
-                                  (1, 128, 8, 32, 32, None)])
+                                  (1, 128, 8, 32, 32, None), (1, 2048, 2, 64, 16, None), (1, 512, 3, 32, 20, None),
+                                  (2, 4096, 1, 64, 8, None)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
