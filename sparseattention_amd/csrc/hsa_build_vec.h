@@ -11,8 +11,11 @@ __device__ __forceinline__ void load_vec(const typename T::storage *p, float (&f
     if constexpr (VEC == 1) {
         f[0] = to_float<T>(p[0]);
     } else {
+        // every operand of a level is read once per launch: streaming hint
         using P = Pack<T, VEC>;
-        P v = *reinterpret_cast<const P *>(p);
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        static_assert(sizeof(P) == 16, "vector path moves 16 bytes per lane");
+        const P v = __builtin_bit_cast(P, __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p)));
 #pragma unroll
         for (int i = 0; i < VEC; ++i) f[i] = to_float<T>(v.e[i]);
     }
