@@ -37,6 +37,23 @@ def test_step_replays_from_a_hip_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
+    # a launch on a capturing stream builds the tree level group by level group (the one-launch
+    # build keeps per-stream arrival counters, and a captured launch may replay on any stream):
+    # the eager runs it is compared with bit for bit take the same route
+    from sparseattention_amd import _lib
+    assert _lib.lib().hsa_build_tree_tune(0, -1) == 0
+    try:
+        _replays_equal_eager(graph, step, mk, q, qp, kp, vp, kfull, vfull, out, N)
+    finally:
+        assert _lib.lib().hsa_build_tree_tune(1, -1) == 0
+    # and the one-launch build agrees with it to the rounding of one multiply-add
+    nodes = kfull[:, N:].clone()
+    sa.build_tree(qp, kp, vp, kfull[:, :N], vfull[:, :N], out=kfull[:, N:], out2=vfull[:, N:])
+    torch.cuda.synchronize()
+    assert (nodes.float() - kfull[:, N:].float()).abs().max() <= 2e-2
+
+
+def _replays_equal_eager(graph, step, mk, q, qp, kp, vp, kfull, vfull, out, N):
     for rep in range(4):
         for buf, rows in ((q, N), (qp, N - 1), (kp, N - 1), (vp, N - 1)):
             buf.copy_(mk(rows))
