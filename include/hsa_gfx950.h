@@ -226,8 +226,9 @@ int hsa_topology_device(int N, int causal, int32_t *idx, uint8_t *mask, int32_t 
 /*
  * Initial span nodes: level-by-level pairwise means of x, each level rounded to
  * the element type.  Replaces generate_span_input_Y
- * (hierarchical_attention/ops/topology.py:153-169) for power-of-two N.
- *   x [B, N, C], y [B, N-1, C]
+ * (hierarchical_attention/ops/topology.py:153-169) for any N >= 2: level l holds N >> l
+ * rows (an unpaired last row of a level has no parent), N - popcount(N) rows in all.
+ *   x [B, N, C], y [B, N - popcount(N), C]  (N-1 rows for a power of two)
  */
 int hsa_span_input_y(const void *x, void *y, int B, int N, int C, int dtype, void *stream);
 
@@ -304,8 +305,8 @@ int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void 
 /*
  * Backward of the initial span nodes (the reference differentiates generate_span_input_Y,
  * hierarchical_attention/ops/topology.py:153-169, through torch autograd):
- *   dx[b, n, :] = sum_{l=1..log2 N} 2^-l * dy[b, level l node n >> l, :]
- *   dy [B, N-1, C], dx [B, N, C]
+ *   dx[b, n, :] = sum over levels l >= 1 with n >> l < N >> l of 2^-l * dy[b, level l node n >> l, :]
+ *   dy [B, N - popcount(N), C], dx [B, N, C]
  */
 int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtype, void *stream);
 

@@ -627,11 +627,18 @@ __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, ty
     const int c = (int)(t % C);
     const int n = (int)((t / C) % N);
     const int b = (int)(t / ((size_t)C * N));
-    const typename T::storage *dy = dY + (size_t)b * (N - 1) * C + c;
+    // level l holds N >> l rows; a leaf under an unpaired row contributes to no level above it
+    int start = 0;
+    for (int l = 1; l <= L; ++l) start += N >> l;
+    const typename T::storage *dy = dY + (size_t)b * start * C + c;
     float acc = 0.f, w = 1.f;
+    start = 0;
     for (int l = 1; l <= L; ++l) {
         w *= 0.5f;
-        acc = fmaf(w, to_float<T>(dy[(size_t)(level_offset(N, l) - N + (n >> l)) * C]), acc);
+        const int rows = N >> l;
+        if ((n >> l) >= rows) break;
+        acc = fmaf(w, to_float<T>(dy[(size_t)(start + (n >> l)) * C]), acc);
+        start += rows;
     }
     dX[t] = from_float<T>(acc);
 }
@@ -820,8 +827,8 @@ int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void 
 int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtype, void *stream) {
     HSA_REQUIRE(dy && dx, "null pointer");
     HSA_REQUIRE(B >= 1 && C >= 1, "bad shape B=%d C=%d", B, C);
-    HSA_REQUIRE(N >= 2 && hsa::ilog2_exact(N) >= 0, "N must be a power of two >= 2 (got %d)", N);
-    const int L = hsa::ilog2_exact(N);
+    HSA_REQUIRE(N >= 2 && N <= (1 << 26), "N must lie in [2, 2^26] (got %d)", N);
+    const int L = hsa::span_levels(N);
     const size_t total = (size_t)B * N * C;
     const unsigned blocks = (unsigned)((total + 255) / 256);
     hipStream_t st = (hipStream_t)stream;

@@ -109,4 +109,18 @@ __host__ __device__ __forceinline__ int level_offset(int N, int l) {
     return l == 0 ? 0 : 2 * N - (N >> (l - 1));
 }
 
+// Rows of the initial span nodes of any leaf count N: level l (l >= 1) holds N >> l rows (an odd
+// row at the end of a level has no partner and no parent); first row of level l within y.
+__host__ __device__ __forceinline__ int span_level_start(int N, int l) {
+    int s = 0;
+    for (int j = 1; j < l; ++j) s += N >> j;
+    return s;
+}
+static inline int span_levels(int N) {
+    int l = 0;
+    while ((N >> (l + 1)) >= 1) ++l;
+    return l;
+}
+static inline int span_rows(int N) { return span_level_start(N, span_levels(N) + 1); }
+
 }  // namespace hsa

@@ -89,9 +89,10 @@ __global__ void span_y_kernel(const typename T::storage *__restrict__ x, size_t 
                               typename T::storage *__restrict__ y, size_t y_bs, int N, int C,
                               int lvl0, int nlev, int B) {
     // src: rows of level lvl0 (lvl0 == 0: x itself; else inside y).  Each thread
-    // takes 2^nlev consecutive source rows of one channel.
+    // takes 2^nlev consecutive source rows of one channel; the last group of a level
+    // whose row count is not a multiple of that is partly filled.
     const int span = 1 << nlev;
-    const int groups = src_rows >> nlev;
+    const int groups = (src_rows + span - 1) >> nlev;
     size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t total = (size_t)B * groups * C;
     if (t >= total) return;
@@ -99,18 +100,22 @@ __global__ void span_y_kernel(const typename T::storage *__restrict__ x, size_t 
     int g = (int)((t / C) % groups);
     int b = (int)(t / ((size_t)C * groups));
     const typename T::storage *src =
-        (lvl0 == 0) ? x + (size_t)b * x_bs : y + (size_t)b * y_bs + (size_t)(level_offset(N, lvl0) - N) * C;
+        (lvl0 == 0) ? x + (size_t)b * x_bs : y + (size_t)b * y_bs + (size_t)span_level_start(N, lvl0) * C;
     float v[32];
 #pragma unroll
     for (int i = 0; i < 32; ++i)
-        if (i < span) v[i] = to_float<T>(src[((size_t)g * span + i) * C + c]);
+        if (i < span) {
+            const int row = g * span + i;
+            v[i] = row < src_rows ? to_float<T>(src[(size_t)row * C + c]) : 0.f;
+        }
     int cnt = span;
 #pragma unroll
     for (int s = 1; s <= 5; ++s) {
         if (s <= nlev) {
             cnt >>= 1;
             int lvl = lvl0 + s;
-            typename T::storage *dst = y + (size_t)b * y_bs + (size_t)(level_offset(N, lvl) - N) * C;
+            const int lvl_rows = src_rows >> s;
+            typename T::storage *dst = y + (size_t)b * y_bs + (size_t)span_level_start(N, lvl) * C;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 if (i < cnt) {
@@ -120,7 +125,8 @@ __global__ void span_y_kernel(const typename T::storage *__restrict__ x, size_t 
                     float hb = to_float<T>(from_float<T>(0.5f * v[2 * i + 1]));
                     float m = ha + hb;
                     typename T::storage r = from_float<T>(m);
-                    dst[((size_t)g * cnt + i) * C + c] = r;
+                    const int row = g * cnt + i;
+                    if (row < lvl_rows) dst[(size_t)row * C + c] = r;
                     v[i] = to_float<T>(r);
                 }
             }
@@ -130,15 +136,16 @@ __global__ void span_y_kernel(const typename T::storage *__restrict__ x, size_t 
 
 template <typename T>
 static int span_y_launch(const void *x, void *y, int B, int N, int C, hipStream_t st) {
-    const int L = ilog2_exact(N);
+    const int L = span_levels(N);
+    const size_t y_rows = (size_t)span_rows(N);
     int lvl = 0, rows = N;
     while (lvl < L) {
         int nlev = L - lvl < 5 ? L - lvl : 5;
-        size_t total = (size_t)B * (rows >> nlev) * C;
+        size_t total = (size_t)B * ((rows + (1 << nlev) - 1) >> nlev) * C;
         int threads = 256;
         unsigned blocks = (unsigned)((total + threads - 1) / threads);
         span_y_kernel<T><<<blocks, threads, 0, st>>>((const typename T::storage *)x, (size_t)N * C, rows,
-                                                     (typename T::storage *)y, (size_t)(N - 1) * C, N,
+                                                     (typename T::storage *)y, y_rows * C, N,
                                                      C, lvl, nlev, B);
         lvl += nlev;
         rows >>= nlev;
@@ -184,7 +191,7 @@ int hsa_topology_device(int N, int causal, int32_t *idx, uint8_t *mask, int32_t 
 int hsa_span_input_y(const void *x, void *y, int B, int N, int C, int dtype, void *stream) {
     HSA_REQUIRE(x && y, "null pointer");
     HSA_REQUIRE(B >= 1 && C >= 1, "bad shape B=%d C=%d", B, C);
-    HSA_REQUIRE(N >= 2 && hsa::ilog2_exact(N) >= 0, "N must be a power of two >= 2 (got %d)", N);
+    HSA_REQUIRE(N >= 2 && N <= (1 << 26), "N must lie in [2, 2^26] (got %d)", N);
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
         case HSA_F32: return hsa::span_y_launch<hsa::F32>(x, y, B, N, C, st);

@@ -92,31 +92,33 @@ class _SpanInputY(torch.autograd.Function):
     def forward(ctx, x):
         B, N, C = x.shape
         x = x.contiguous()
-        y = torch.empty((B, N - 1, C), dtype=x.dtype, device=x.device)
+        y = torch.empty((B, N - bin(N).count("1"), C), dtype=x.dtype, device=x.device)
         with torch.cuda.device(x.device):
             rc = _lib.lib().hsa_span_input_y(_lib.ptr(x), _lib.ptr(y), B, N, C, _lib.dtype_code(x),
                                              _lib.stream_of(x))
         _lib.check(rc, "hsa_span_input_y")
+        ctx.leaves = N
         return y
 
     @staticmethod
     def backward(ctx, dy):
         B, M, C = dy.shape
         dy = dy.contiguous()
-        dx = torch.empty((B, M + 1, C), dtype=dy.dtype, device=dy.device)
+        N = ctx.leaves
+        dx = torch.empty((B, N, C), dtype=dy.dtype, device=dy.device)
         with torch.cuda.device(dy.device):
-            rc = _lib.lib().hsa_span_input_y_bwd(_lib.ptr(dy), _lib.ptr(dx), B, M + 1, C, _lib.dtype_code(dy),
+            rc = _lib.lib().hsa_span_input_y_bwd(_lib.ptr(dy), _lib.ptr(dx), B, N, C, _lib.dtype_code(dy),
                                                  _lib.stream_of(dy))
         _lib.check(rc, "hsa_span_input_y_bwd")
         return dx
 
 
 def generate_span_input_Y(x: torch.Tensor) -> Optional[torch.Tensor]:
-    """Initial span nodes: pairwise means level by level, [B, N, C] -> [B, N-1, C]."""
+    """Initial span nodes: pairwise means level by level, [B, N, C] -> [B, N-1, C] (any N: an unpaired
+    last row of a level has no parent, N - popcount(N) rows in all)."""
     B, N, C = x.shape
     if N < 2:
         return None
-    assert (N & (N - 1)) == 0, "sequence length must be a power of 2"
     _lib.require_gpu(x)
     _lib.dtype_code(x)
     return _SpanInputY.apply(x)

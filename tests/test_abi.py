@@ -87,7 +87,7 @@ def test_attention_argument_checks_on_host():
     assert lib.hsa_attn_fwd(one, one, one, None, None, one, None, 1, 16, 31, 1, 64, 4, 1, 1, 7, 0, None) == -22
     assert lib.hsa_build_parents_fwd(None, one, one, one, one, one, None, 1, 1, 1, 8, 0, 0, 0, 0, 0, 0, 0, None) == -22
     assert lib.hsa_build_tree_fwd(one, one, one, one, one, one, None, 1, 12, 1, 8, 0, 0, 0, 0, 0, 0, 0, 0, None) == -22
-    assert lib.hsa_span_input_y(one, one, 1, 6, 4, 0, None) == -22
+    assert lib.hsa_span_input_y(one, one, 1, 1, 4, 0, None) == -22
 
 
 def test_ops_refuse_cpu_tensors_instead_of_falling_back():
