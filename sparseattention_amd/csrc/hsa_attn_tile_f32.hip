@@ -32,7 +32,9 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int TQ = 16;            // queries per block
 // wavefronts per workgroup: two per SIMD (256 registers each) where the variant fits, so that one
 // wavefront's matrix work overlaps the other's loads; else one per SIMD (up to 512 registers)
-template <int D, int NBW, bool CAUSAL> constexpr bool f32_fits_two_per_simd() { return D <= 32 || (CAUSAL && NBW <= 1); }
+template <int D, int NBW, bool CAUSAL> constexpr bool f32_fits_two_per_simd() { return D <= 32 || (D <= 64 && CAUSAL && NBW <= 1); }
+// longest strip whose operands stay in registers
+template <int D, int NBW, bool CAUSAL> constexpr int f32_max_strip() { return D <= 64 ? 4 : ((CAUSAL && NBW <= 1) ? 2 : 1); }
 constexpr int F32_MAX_LEVELS = 22;
 constexpr int F32_MAX_NBW = 2;
 constexpr float NEG_INF_F = -__builtin_inff();
@@ -344,13 +346,24 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
 template <int D, int NBW, bool CAUSAL, int WPB>
 int launch_wpb(const TileF32Params &p, int sb, hipStream_t st) {
     const int nwg = (p.n_units + WPB - 1) / WPB;
-    switch (sb) {
-        case 1: attn_tile_f32_kernel<D, NBW, CAUSAL, 1, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
-        case 2: attn_tile_f32_kernel<D, NBW, CAUSAL, 2, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
-        case 4: attn_tile_f32_kernel<D, NBW, CAUSAL, 4, WPB><<<nwg, WPB * 64, 0, st>>>(p); break;
-        default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
+    constexpr int MAXSB = f32_max_strip<D, NBW, CAUSAL>();
+    if (sb == 1) {
+        attn_tile_f32_kernel<D, NBW, CAUSAL, 1, WPB><<<nwg, WPB * 64, 0, st>>>(p);
+        return check_launch("attn_tile_f32_kernel");
     }
-    return check_launch("attn_tile_f32_kernel");
+    if constexpr (MAXSB >= 2) {
+        if (sb == 2) {
+            attn_tile_f32_kernel<D, NBW, CAUSAL, 2, WPB><<<nwg, WPB * 64, 0, st>>>(p);
+            return check_launch("attn_tile_f32_kernel");
+        }
+    }
+    if constexpr (MAXSB >= 4) {
+        if (sb == 4) {
+            attn_tile_f32_kernel<D, NBW, CAUSAL, 4, WPB><<<nwg, WPB * 64, 0, st>>>(p);
+            return check_launch("attn_tile_f32_kernel");
+        }
+    }
+    return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built for this variant", sb);
 }
 
 template <int D, int NBW, bool CAUSAL>
@@ -381,7 +394,7 @@ void attn_tile_knobs_sb_swizzle(int *sb, int *swizzle);  // hsa_attn_tile.hip
 
 bool attn_tile_f32_eligible(int N, int M, int D, int L, int R, bool canonical, bool want_weights) {
     if (!canonical || want_weights) return false;
-    if (D != 32 && D != 64) return false;
+    if (D != 32 && D != 64 && D != 128) return false;
     if (N < TQ || ilog2_exact(N) != L || L > F32_MAX_LEVELS) return false;
     if (M < 2 * N - 1) return false;
     return (R + TQ - 1) / TQ <= F32_MAX_NBW;
@@ -403,6 +416,7 @@ int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *ou
     attn_tile_knobs_sb_swizzle(&forced_sb, &swizzle);
     if (forced_sb) sb = forced_sb;
     if (!causal && nbw >= 2 && sb > 2) sb = 2;  // five leaf blocks: registers
+    if (D == 128) sb = sb > 1 && causal && nbw <= 1 ? 2 : 1;
     while (sb > NB) sb >>= 1;
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;
@@ -411,6 +425,7 @@ int attn_tile_f32_dispatch(const void *q, const void *k, const void *v, void *ou
     p.xcd_swizzle = swizzle;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
     if (D == 32) return launch_d<32>(p, nbw, causal != 0, sb, st);
+    if (D == 128) return launch_d<128>(p, nbw, causal != 0, sb, st);
     return launch_d<64>(p, nbw, causal != 0, sb, st);
 }
 

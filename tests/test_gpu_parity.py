@@ -619,7 +619,10 @@ def test_attention_random_shapes(seed):
 
 
 F32_TILE_CASES = [(1, 16, 2, 64, 3), (2, 64, 3, 64, 16), (1, 256, 4, 32, 8), (2, 128, 2, 64, 20), (1, 512, 5, 32, 32),
-                  (1, 64, 2, 64, 0), (2, 1024, 8, 64, 16)]
+                  (1, 64, 2, 64, 0), (2, 1024, 8, 64, 16),
+                  # head size 128: strips of one block (two where the window is causal and at most one block wide)
+                  (1, 16, 2, 128, 3), (2, 256, 3, 128, 16), (1, 128, 2, 128, 32), (1, 2048, 8, 128, 16),
+                  (1, 64, 1, 128, 0)]
 
 
 @pytest.mark.parametrize("case", F32_TILE_CASES)
