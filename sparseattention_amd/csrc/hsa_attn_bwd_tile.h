@@ -642,8 +642,8 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
 // root, right-hand nodes when causal, rows past 2N-1) get zeros.  One thread per (batch, row,
 // head, channel).  lg_sb = log2 of the blocks per strip of the query pass.
 template <typename T>
-__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, uint16_t *__restrict__ dk,
-                                            uint16_t *__restrict__ dv, int B, int N, int M, int H, int D, int L,
+__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
+                                            typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D, int L,
                                             int causal, int first_row, int lg_sb) {
     const size_t per_b = (size_t)(M - first_row) * H * D;
     const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;

@@ -644,7 +644,13 @@ __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, ty
 }
 
 // ---------------------------------------------------------------- tile backward dispatch
+bool attn_bwd_tile_f32_eligible(int N, int M, int D, int L, int R);  // hsa_attn_bwd_tile_f32.hip
+int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
+                               void *dv, float *ws, int B, int N, int M, int H, int D, int L, int R, int causal,
+                               hipStream_t st);
+
 static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype) {
+    if (dtype == HSA_F32) return attn_bwd_tile_f32_eligible(N, M, D, L, R);
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
@@ -759,6 +765,8 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
     if (algo == HSA_ATTN_TILE && !tile_ok)
         return hsa::fail(HSA_ERR_UNSUPPORTED, "tile backward not available for N=%d D=%d L=%d R=%d dtype=%d", N, D, L, R, dtype);
     if (tile_ok && algo != HSA_ATTN_GATHER) {
+        if (dtype == HSA_F32)
+            return hsa::attn_bwd_tile_f32_dispatch(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);
         if (dtype == HSA_BF16)
             return hsa::attn_bwd_tile_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);
         return hsa::attn_bwd_tile_typed<hsa::F16>(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);

@@ -9,6 +9,7 @@ import torch
 
 import oracle
 import sparseattention_amd as sa
+from sparseattention_amd import _lib
 from sparseattention_amd.ops import functional as fn
 
 pytestmark = pytest.mark.gpu
@@ -809,6 +810,40 @@ def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
     _grad_close(dq, qr.grad, dtype, "dQ gather")
     _grad_close(dk, kr.grad, dtype, "dK gather")
     _grad_close(dv, vr.grad, dtype, "dV gather")
+
+
+F32_BWD_TILE_CASES = [(1, 16, 2, 64, 3), (2, 64, 3, 64, 16), (1, 256, 4, 32, 8), (2, 128, 2, 32, 16), (1, 64, 2, 64, 0),
+                      (1, 1024, 8, 64, 16), (1, 4096, 2, 32, 12), (2, 128, 1, 64, 7)]
+
+
+@pytest.mark.parametrize("case", F32_BWD_TILE_CASES)
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_backward_tile_fp32(case, causal):
+    """fp32 gradients on the fp32 matrix instructions: against autograd through the fp64 oracle and
+    against the per-query gather formulation."""
+    B, N, H, D, R = case
+    q, k, v = make_qkv(B, N, H, D, torch.float32, seed=5 * N + R + D)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(4))
+    o = oracle.topology_tables(N, causal)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"] if causal else None, R).backward(go.double())
+    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), R, causal)
+    dq, dk, dv = fn.attention_backward(*args, algo="tile")
+    for name, got, want in (("dQ", dq, qr.grad), ("dK", dk, kr.grad), ("dV", dv, vr.grad)):
+        _grad_close(got, want, torch.float32, name)
+    gq, gk, gv = fn.attention_backward(*args, algo="gather")
+    for got, other in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (got - other).abs().max() <= 4e-5 * max(1.0, float(other.abs().max()))
+
+
+def test_attention_backward_tile_fp32_limits():
+    """Shapes outside the fp32 tile backward are refused with algo="tile" and run on the gather kernels otherwise."""
+    q, k, v = make_qkv(1, 64, 2, 64, torch.float32, seed=2)
+    go = torch.randn(1, 64, 2, 64)
+    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), 20, True)
+    with pytest.raises(_lib.HsaError):
+        fn.attention_backward(*args, algo="tile")
+    fn.attention_backward(*args)
 
 
 def test_attention_backward_rejects_unknown_tables():
