@@ -9,10 +9,12 @@
 //      and stores dQ plus two numbers per (query, head): the log2-domain log-sum-exp and delta.
 //      The tree key blocks are also evaluated in the other orientation (S[query, slot]), which
 //      puts the queries into the MFMA contraction: dK^T[ch, slot] = Q^T . dS, dV^T = dO^T . P.
-//      Nodes of levels 1..3 are attended only from inside the block: their rows are final and
-//      written directly.  A node of level l >= 4 collects from the 2^(l-4) blocks under its
-//      sibling: every block stores its fp32 partial row per level, and a small reduction kernel
-//      sums each node's contiguous run of blocks (deterministic, no atomics).
+//      Nodes of levels 1..4 are attended only from inside the block: their rows are final and
+//      written directly.  A node of level l >= 5 collects from the 2^(l-4) blocks under its
+//      sibling: a wavefront that walks a strip of four blocks finishes level 5 itself and sums
+//      the levels above over its strip; what is left is stored as fp32 partial rows (per strip
+//      and level >= 6, or per block and level >= 5 for strips of one block), and a small
+//      reduction kernel sums each node's contiguous run (deterministic, no atomics).
 //  (B) key-stationary, one wavefront per (batch, head, 16-leaf key block): loops over the query
 //      blocks whose window reaches the key block, rebuilds P and dS from the saved statistics
 //      and accumulates dK^T = Q^T . dS, dV^T = dO^T . P in registers.  Every leaf row of dK / dV
@@ -117,8 +119,9 @@ struct BwdTile {
 // and the partial rows it collects are summed over the strip's blocks before they are written.
 // The next block's rows are requested while the current block is computed.
 //
-// Partial rows (fp32): levels 4 and 5 per query block, [2][B][N/16][H][2][D] (dK then dV);
-// levels >= 6 per strip, [2][B][N/16/SB][H][L-6][D], right behind.
+// Partial rows (fp32): level 5 per query block when SB == 1, entry 1 of [2][B][N/16][H][2][D]
+// (dK then dV; entry 0 and, for longer strips, the whole area stay unused); levels >= 6 per
+// strip, [2][B][N/16/SB][H][L-6][D], right behind.
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(BWD_WPB * 64)
 attn_bwd_tile_query_kernel(BwdTileParams p) {
@@ -129,6 +132,8 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
     constexpr int LDS_SLOTS = 4;
     __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
+    // level-5 rows (dK, dV) of an even block, kept until the odd block of the pair adds its own
+    __shared__ __align__(16) float carry_mem[SB > 1 ? BWD_WPB * 2 * D : 4];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = blockIdx.x * BWD_WPB + wave;
@@ -136,6 +141,7 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
     const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
+    float *carry = carry_mem + (SB > 1 ? wave * 2 * D : 0);
 
     const int N = p.N, L = p.L, R = p.R, H = p.H;
     const int NB = N / TILE_Q, NS = NB / SB;
@@ -415,21 +421,29 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
                     tk[j] = M_::k16(QT[j], dk, z);
                     tv[j] = M_::k16(GT[j], pk, z);
                 }
-                // slots 0..13 (levels 1..3) are complete: rows written directly
-                bt.put_result(0, tk, 1.0f);
-                bt.put_result(1, tv, 1.0f);
+                // A level-5 node collects from the two blocks under its sibling.  In a strip both
+                // are this wavefront's: the even block parks its row, the odd block adds it and
+                // the sum is final.  A strip of one block stores a partial row instead.
+                bool five_final = false;
+                if constexpr (SB > 1) {
+                    if (r16 == 15) {
 #pragma unroll
-                for (int i = 0; i < NLD; ++i) {
-                    const int sl = i * RPI + lrow;
-                    if (sl < 14 && t_row[i] >= 0) {
-                        *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
-                        *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
+                        for (int j = 0; j < NJ; ++j) {
+                            const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                            if (it & 1) {
+                                const f32x4 ck = *reinterpret_cast<const f32x4 *>(carry + ch);
+                                const f32x4 cv = *reinterpret_cast<const f32x4 *>(carry + D + ch);
+                                tk[j] += ck;
+                                tv[j] += cv;
+                            } else {
+                                *reinterpret_cast<f32x4 *>(carry + ch) = tk[j];
+                                *reinterpret_cast<f32x4 *>(carry + D + ch) = tv[j];
+                            }
+                        }
                     }
-                }
-                // levels 4 and 5 collect from one or two blocks: this block's partial rows
-                const int lvl = r16 >= 14 ? 4 + (r16 - 14) : -1;
-                if (lvl >= 4 && lvl < L) {
-                    const size_t po = ((((size_t)b * NB + blk) * H + h) * 2 + (lvl - 4)) * D;
+                    five_final = (it & 1) != 0;
+                } else if (r16 == 15 && 5 < L) {
+                    const size_t po = ((((size_t)b * NB + blk) * H + h) * 2 + 1) * D;
                     float *pkp = p.partial + po;
                     float *pvp = p.partial + (size_t)p.B * NB * H * 2 * D + po;
 #pragma unroll
@@ -437,6 +451,18 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
                         const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
                         *reinterpret_cast<f32x4 *>(pkp + ch) = tk[j];
                         *reinterpret_cast<f32x4 *>(pvp + ch) = tv[j];
+                    }
+                }
+                // slots 0..14 (levels 1..4) are attended from inside the block only: rows written
+                // directly, and so is the finished level-5 row
+                bt.put_result(0, tk, 1.0f);
+                bt.put_result(1, tv, 1.0f);
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int sl = i * RPI + lrow;
+                    if ((sl < 15 || five_final) && t_row[i] >= 0) {
+                        *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
+                        *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
                     }
                 }
             } else {
@@ -637,8 +663,9 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
     }
 }
 
-// Rows of tree levels >= 4 (and anything above row 2N-2): node (l, p) sums the partial rows of the
-// query blocks (levels 4, 5) or strips (levels >= 6) under its sibling; nodes nobody attends (the
+// Rows from first_row on (a level the query pass left unfinished, up to anything above row 2N-2):
+// node (l, p) sums the partial rows of the query blocks (levels 4, 5) or strips (levels >= 6)
+// under its sibling; nodes nobody attends (the
 // root, right-hand nodes when causal, rows past 2N-1) get zeros.  One thread per (batch, row,
 // head, channel).  lg_sb = log2 of the blocks per strip of the query pass.
 template <typename T>

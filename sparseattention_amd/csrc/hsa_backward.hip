@@ -690,7 +690,10 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
            : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
                      : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
     if (rc != HSA_OK) return rc;
-    const int first = level_offset(N, 4);
+    // the query pass finished levels 1..4 (1..5 when it walked strips); the root row and the rows
+    // past 2N-1 are the reduction's in any case
+    int first = level_offset(N, sb == 4 ? 6 : 5);
+    if (first > 2 * N - 2) first = 2 * N - 2;
     const size_t n_fin = (size_t)B * (M - first) * H * D;
     if (n_fin) {
         attn_bwd_tile_reduce_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
