@@ -117,13 +117,15 @@ struct BwdTile {
 // leaf key / value operands slide along the strip in registers (each leaf row is fetched once per
 // strip), the far tree block (levels >= 6, the same nodes for the whole strip) is fetched once,
 // and the partial rows it collects are summed over the strip's blocks before they are written.
-// The next block's rows are requested while the current block is computed.
+// A block's rows are requested when its turn comes: holding the next block's rows in registers
+// as well would cost the second wavefront per SIMD (more than 256 registers at D = 64), and two
+// wavefronts that cover each other's waits are worth more than the prefetch.
 //
 // Partial rows (fp32): level 5 per query block when SB == 1, entry 1 of [2][B][N/16][H][2][D]
 // (dK then dV; entry 0 and, for longer strips, the whole area stay unused); levels >= 6 per
 // strip, [2][B][N/16/SB][H][L-6][D], right behind.
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
-__global__ void __launch_bounds__(BWD_WPB * 64)
+__global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1)))
 attn_bwd_tile_query_kernel(BwdTileParams p) {
     using BT = BwdTile<T, D>;
     using M_ = Mma<T>;
@@ -221,7 +223,7 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
 
     // everything the first block needs is requested before anything is consumed
     u32x4_t Kc[NKB][KS], Vc[NKB][KS];
-    Stage st[SB];
+    Stage sg;
     {
         u32x4_t rKu[NLD], rVu[NLD], rKh[NKL][NLD], rVh[NKL][NLD];
 #pragma unroll
@@ -234,7 +236,7 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
             load_block(Kb, leaf_row0(blk0 - NBW + c), rKh[c]);
             load_block(Vb, leaf_row0(blk0 - NBW + c), rVh[c]);
         }
-        request(st[0], blk0);
+        request(sg, blk0);
         bt.put(2, rKu);
         bt.put(3, rVu);
         bt.get(2, Kc[NKL + 1]);
@@ -256,8 +258,8 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     for (int it = 0; it < SB; ++it) {
         const int blk = blk0 + it;
         const int q0 = blk * TILE_Q;
-        Stage &sg = st[it];
-        // rows -> operand pieces; then the next block's rows are requested
+        if (it > 0) request(sg, blk);
+        // rows -> operand pieces
         u32x4_t Qf[KS], Gf[KS];
         bt.put(0, sg.q);
         bt.put(1, sg.g);
@@ -271,7 +273,6 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
         bt.put(3, sg.vt);
         bt.get(2, Kc[NKL]);
         bt.get(3, Vc[NKL]);
-        if (it + 1 < SB) request(st[it + 1 < SB ? it + 1 : it], blk + 1);
 
         // liveness of the near block and of the leaf blocks for this query block
         int t_row[NLD];
