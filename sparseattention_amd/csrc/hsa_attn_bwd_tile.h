@@ -41,11 +41,19 @@ struct BwdTileParams {
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 
-// Query blocks (key blocks) one wavefront of the backward passes walks: 4 where the operands that
-// slide along the strip (leaf blocks in the query pass, query blocks in the key pass: NBW+1 when
-// causal, 2 NBW+1 otherwise) fit the registers, else 1.
-constexpr int bwd_strip_blocks(int D, int nbw, bool causal) {
+// Blocks one wavefront walks.  Key pass: 4 where the query blocks that slide along the strip in
+// operand form (NBW+1 when causal, 2 NBW+1 otherwise) and the next block's rows fit the registers,
+// else 1.  Query pass: 4 in every variant (1 only for sequences whose block count is no multiple
+// of four).
+constexpr int bwd_key_strip(int D, int nbw, bool causal) {
     return ((causal ? nbw + 1 : 2 * nbw + 1) <= 3 && D <= 64) ? 4 : 1;
+}
+constexpr int BWD_QUERY_STRIP = 4;
+// Wavefronts per SIMD the query pass is compiled for: two (256 registers) where that holds its
+// operands without spilling, which a strip with five sliding leaf blocks at D = 64 and every
+// variant at D = 128 do not.
+constexpr int bwd_query_waves(int D, int nkl, int sb) {
+    return (D <= 32 || (D <= 64 && (nkl <= 3 || sb == 1))) ? 2 : 1;
 }
 
 template <typename T, int D>
@@ -125,7 +133,8 @@ struct BwdTile {
 // (dK then dV; entry 0 and, for longer strips, the whole area stay unused); levels >= 6 per
 // strip, [2][B][N/16/SB][H][L-6][D], right behind.
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
-__global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(D <= 64 ? 2 : 1)))
+__global__ void __launch_bounds__(BWD_WPB * 64)
+__attribute__((amdgpu_waves_per_eu(bwd_query_waves(D, CAUSAL ? NBW + 1 : 2 * NBW + 1, SB))))
 attn_bwd_tile_query_kernel(BwdTileParams p) {
     using BT = BwdTile<T, D>;
     using M_ = Mma<T>;

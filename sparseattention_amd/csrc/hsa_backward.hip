@@ -20,7 +20,7 @@
 namespace hsa {
 
 template <typename T, int D>
-int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb, hipStream_t st);
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sbq, int sbk, hipStream_t st);
 
 // ---------------------------------------------------------------- parent build
 template <typename T, int VEC> struct BPack { typename T::storage e[VEC]; };
@@ -685,10 +685,11 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.scale_log2e = 1.4426950408889634f * p.scale;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     const int NB = N / TILE_Q;
-    const int sb = NB % 4 == 0 ? bwd_strip_blocks(D, nbw, causal != 0) : 1;
-    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, st)
-           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
-                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
+    const int sb = NB % 4 == 0 ? BWD_QUERY_STRIP : 1;                               // query pass
+    const int sbk = NB % 4 == 0 ? bwd_key_strip(D, nbw, causal != 0) : 1;           // key pass
+    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, sbk, st)
+           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, sbk, st)
+                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, sbk, st);
     if (rc != HSA_OK) return rc;
     // the query pass finished levels 1..4 (1..5 when it walked strips); the root row and the rows
     // past 2N-1 are the reduction's in any case
