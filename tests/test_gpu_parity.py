@@ -675,7 +675,9 @@ def test_tile_is_the_default_for_the_headline_shape():
     from sparseattention_amd import _lib
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 1, 0) == 1
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_F32, 1, 0) == 1
-    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 128, 11, 16, _lib.HSA_F32, 1, 0) == 0
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 128, 11, 16, _lib.HSA_F32, 1, 0) == 1
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 48, 11, 16, _lib.HSA_F32, 1, 0) == 0
+    assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 128, 11, 16, _lib.HSA_F32, 1, 1) == 0
     assert _lib.lib().hsa_attn_fwd_uses_tile(2048, 4095, 8, 64, 11, 16, _lib.HSA_BF16, 0, 0) == 0
 
 
