@@ -315,10 +315,25 @@ def step_bytes(B, H, N, D, attention_only):
     return b
 
 
+def between_events(torch, stream, K, launch):
+    """Average time of K calls of `launch(i)` between one pair of events on `stream`."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for i in range(K):
+        launch(i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / K
+
+
 def kernel_times(torch, lib, hip, prob, stream, st, K, with_tree):
-    """Average duration of the span-attention kernel over K steps run one after the other on one
-    stream, every attention dispatch carrying its own pair of HIP events; and the average time
-    of K tree builds between one pair of events on the launch stream."""
+    """Durations on one stream, inputs rotated as in the timed steps:
+      b2b   K span-attention launches one after the other between one pair of events: the average
+            launch duration (an upper bound of the kernel's own: the launch gaps are inside);
+      attn  the K steps once more with every attention dispatch carrying its own pair of HIP
+            events (sorted); such a dispatch reads about 1 us longer than the same kernel in the
+            rocprofv3 trace and than b2b;
+      tree  K tree builds between one pair of events."""
     n = len(prob.sets)
     targs = [prob.tree_args(s, st) for s in prob.sets]
     aargs = [prob.attn_args(s, st) for s in prob.sets]
@@ -334,16 +349,11 @@ def kernel_times(torch, lib, hip, prob, stream, st, K, with_tree):
     for a, b in kev:
         hip.free(a)
         hip.free(b)
+    b2b_ms = between_events(torch, stream, K, lambda i: lib.hsa_attn_fwd(*aargs[i % n]))
     tree_ms = None
     if with_tree:
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for i in range(K):
-            lib.hsa_build_tree_fwd(*targs[i % n])
-        e1.record(stream)
-        torch.cuda.synchronize()
-        tree_ms = e0.elapsed_time(e1) / K
-    return attn, tree_ms
+        tree_ms = between_events(torch, stream, K, lambda i: lib.hsa_build_tree_fwd(*targs[i % n]))
+    return {"attn": attn, "b2b": b2b_ms, "tree": tree_ms}
 
 
 def wall_ms_per_step(torch, lib, prob, st_list, K, with_tree):
@@ -375,14 +385,17 @@ def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
     for _ in range(2):
         wall_ms_per_step(torch, lib, prob, [st], min(K, 10), True)
     step_ms = wall_ms_per_step(torch, lib, prob, [st], K, True)
-    attn, tree_ms = kernel_times(torch, lib, hip, prob, stream, st, K, True)
-    a_ms = sum(attn) / len(attn)
+    kt = kernel_times(torch, lib, hip, prob, stream, st, K, True)
+    attn, tree_ms, a_ms = kt["attn"], kt["tree"], kt["b2b"]
+    e_ms = sum(attn) / len(attn)
     rec = {"workload": desc if causal else desc.replace("causal", "not causal"),
            "head_queries_per_step": prob.head_queries, "buffer_sets_rotated": nsets, "steps": K,
-           "attn_kernel_avg_ms": a_ms, "attn_kernel_median_ms": attn[len(attn) // 2],
+           "attn_back_to_back_avg_ms": a_ms, "attn_in_step_dispatch_event_avg_ms": e_ms,
+           "attn_in_step_dispatch_event_median_ms": attn[len(attn) // 2],
            "attn_algorithmic_bytes": prob.attn_bytes,
            "attn_GBps": prob.attn_bytes / (a_ms * 1e-3) / 1e9,
            "attn_frac_of_hbm_peak": prob.attn_bytes / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+           "attn_frac_of_hbm_peak_in_step_events": prob.attn_bytes / (e_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "tree_build_avg_launch_ms": tree_ms, "tree_algorithmic_bytes": prob.tree_bytes,
            "tree_GBps": prob.tree_bytes / (tree_ms * 1e-3) / 1e9,
            "tree_frac_of_hbm_peak": prob.tree_bytes / (tree_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -447,22 +460,15 @@ def main():
     wall_ms_per_step(torch, lib, prob, [st], min(args.warmup, 10), with_tree)
     serial_ms_per_step = wall_ms_per_step(torch, lib, prob, [st], K, with_tree)
 
-    # --- duration of the dominant kernel: the same K steps once more on one stream, every
-    #     attention dispatch carrying its own pair of HIP events (kept out of the region above
-    #     because an event-carrying dispatch costs the step about 3 us of completion handling);
-    #     and K tree builds between one pair of events -----------------------------------------
-    attn_kernel_ms, tree_b2b_ms = kernel_times(torch, lib, hip, prob, stream, st, K, with_tree)
-    attn_avg_ms = sum(attn_kernel_ms) / K
-
-    # --- K attention launches between one pair of events (kernel durations plus launch gaps) ---
-    aargs = [prob.attn_args(s, st) for s in prob.sets]
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(K):
-        lib.hsa_attn_fwd(*aargs[i % nsets])
-    e1.record(stream)
-    torch.cuda.synchronize()
-    attn_b2b_ms = e0.elapsed_time(e1) / K
+    # --- duration of the dominant kernel, on one stream with the same rotation of inputs: K
+    #     attention launches between one pair of events (the figure of the roofline object), the
+    #     K steps once more with an event pair on every attention dispatch (kept out of the timed
+    #     region: such a dispatch costs the step about 3 us of completion handling), K tree
+    #     builds and K whole steps between one pair of events each ------------------------------
+    kt = kernel_times(torch, lib, hip, prob, stream, st, K, with_tree)
+    attn_kernel_ms, tree_b2b_ms, attn_b2b_ms = kt["attn"], kt["tree"], kt["b2b"]
+    attn_avg_ms = attn_b2b_ms
+    attn_event_avg_ms = sum(attn_kernel_ms) / K
 
     # --- backward of the span attention (next-row kernel), same rotation of inputs ----------------
     P = lambda t: ctypes.c_void_p(t.data_ptr())
@@ -518,15 +524,17 @@ def main():
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes_per_launch": attn_bytes, "avg_launch_ms": attn_avg_ms,
-                     "median_launch_ms": attn_kernel_ms[K // 2], "min_launch_ms": attn_kernel_ms[0],
-                     "timing": "HIP events attached to each attention dispatch (kernel begin/end) over a repeat of the K timed steps, one after the other on one stream"},
+                     "timing": "K launches of the kernel one after the other on one stream between one pair of HIP events, inputs rotated as in the timed steps (launch gaps included: an upper bound of the kernel's duration)",
+                     "per_dispatch_events": {"avg_ms": attn_event_avg_ms, "median_ms": attn_kernel_ms[K // 2],
+                                             "min_ms": attn_kernel_ms[0],
+                                             "frac": attn_bytes / (attn_event_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                             "timing": "the K steps once more, one stream, a HIP event pair attached to every attention dispatch (reads about 1 us more than the same dispatch in the rocprofv3 kernel trace)"}},
         "detail": {"single_stream_ms_per_step": serial_ms_per_step,
                    "single_stream_head_queries_per_s": head_queries / (serial_ms_per_step * 1e-3),
                    "step_algorithmic_bytes": step_algorithmic,
                    "step_GBps_two_streams": step_algorithmic / (ms_per_step * 1e-3) / 1e9,
                    "step_frac_of_hbm_peak_two_streams": step_algorithmic / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                    "attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
-                   "attn_back_to_back_ms_incl_launch_gaps": attn_b2b_ms,
                    "attn_backward_avg_ms": attn_bwd_ms,
                    "attn_backward_algorithmic_bytes": E * B * H * D * (2 * N + 2 * M + N + 2 * M)},
     }
@@ -551,11 +559,12 @@ def main():
         ao = Problem(torch, _lib, B, H, N, D, R, scale, causal, ns, 1, iid_nodes=True)
         wall_ms_per_step(torch, lib, ao, [st], 20, False)
         ao_ms = wall_ms_per_step(torch, lib, ao, [st], K, False)
-        ao_k, _ = kernel_times(torch, lib, hip, ao, stream, st, K, False)
+        ao_k = kernel_times(torch, lib, hip, ao, stream, st, K, False)
         result["detail"]["attention_only_one_stream"] = {
             "ms_per_launch_wall_clock": ao_ms, "head_queries_per_s_wall_clock": head_queries / (ao_ms * 1e-3),
             "frac_of_hbm_peak_wall_clock": attn_bytes / (ao_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-            "kernel_avg_ms": sum(ao_k) / K, "buffer_sets_rotated": ns}
+            "kernel_avg_ms_between_events": ao_k["b2b"], "dispatch_event_avg_ms": sum(ao_k["attn"]) / K,
+            "buffer_sets_rotated": ns}
         del ao
         torch.cuda.empty_cache()
         kb = min(K, 60)
