@@ -111,6 +111,11 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
     using P = VPack<T, VEC>;
     constexpr int NC = 1 << TL;
     constexpr int PB = (int)sizeof(P);  // 16 bytes
+    // Node rows leave with the streaming hint in the small-workgroup variants, i.e. when the
+    // launch leaves half the chip's wavefront slots empty: there it takes 2-3 us off the launch
+    // (measured at B16 N512 .. B2 N4096, 8 heads of 64), while at 512 threads the launch gains
+    // nothing and the span attention that follows loses the node rows the memory-side cache kept.
+    constexpr bool STREAM = THREADS <= 256;
     extern __shared__ __align__(16) unsigned char tree_lds[];
     unsigned char *bufX = tree_lds;                       // 2 * THREADS pieces
     unsigned char *bufY = tree_lds + 2 * THREADS * PB;    // THREADS pieces
@@ -210,8 +215,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                 lvl[i].e[e] = from_float<T>(w0 * to_float<T>(rv[i].e[e]) + w1 * to_float<T>(rcv[2 * i].e[e]) +
                                             w2 * to_float<T>(rcv[2 * i + 1].e[e]));
             const size_t row = node_row(1, sub * (NC / 2) + i);
-            store_node<0>(Out + row, lvl[i]);
-            if (Out2) store_node<1>(Out2 + row, lvl[i]);
+            store_node<STREAM>(Out + row, lvl[i]);
+            if (Out2) store_node<STREAM>(Out2 + row, lvl[i]);
         }
         // levels 2..TL
 #pragma unroll
@@ -225,8 +230,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                                                 a.scale);
                     const size_t row = node_row(j, sub * np + i);
                     if (j == TL && lgS == 0 && lg_wpb > 0) publish_piece(Out + row, r);
-                    else store_node<0>(Out + row, r);
-                    if (Out2) store_node<1>(Out2 + row, r);
+                    else store_node<STREAM>(Out + row, r);
+                    if (Out2) store_node<STREAM>(Out2 + row, r);
                     lvl[i] = r;
                 }
             }
@@ -250,8 +255,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                 const P r = combine<T, VEC>(bq[j - 1], bk[j - 1], bv[j - 1], c0, c1, G, a.scale);
                 const size_t row = node_row(TL + j, ((wg << lgS) >> j) + p_local);
                 if (j == lgS && lg_wpb > 0) publish_piece(Out + row, r);  // the workgroup's node
-                else store_node<0>(Out + row, r);
-                if (Out2) store_node<1>(Out2 + row, r);
+                else store_node<STREAM>(Out + row, r);
+                if (Out2) store_node<STREAM>(Out2 + row, r);
                 if (j < lgS) *reinterpret_cast<P *>(dst + (size_t)threadIdx.x * PB) = r;
             }
             if (j < lgS) lds_barrier();
@@ -316,8 +321,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                     const P r = combine<T, VEC>(cq[pass], ckk[pass], cvv[pass], ch0[pass], ch1[pass], G, a.scale);
                     const size_t row = node_row(level + 1, (grp << (g - 1)) + p);
                     if (g == 1 && lg_width > g) publish_piece(Out + row, r);  // read by the next stage
-                    else store_node<0>(Out + row, r);
-                    if (Out2) store_node<1>(Out2 + row, r);
+                    else store_node<STREAM>(Out + row, r);
+                    if (Out2) store_node<STREAM>(Out2 + row, r);
                     if (g > 1) *reinterpret_cast<P *>(bufX + (((size_t)u << lgG) + gl) * PB) = r;
                 }
             }
@@ -336,8 +341,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                     const P r = combine<T, VEC>(cq[j], ckk[j], cvv[j], c0, c1, G, a.scale);
                     const size_t row = node_row(level + j, (grp << (g - j)) + p_local);
                     if (j == g && lg_width > g) publish_piece(Out + row, r);  // read by the next stage
-                    else store_node<0>(Out + row, r);
-                    if (Out2) store_node<1>(Out2 + row, r);
+                    else store_node<STREAM>(Out + row, r);
+                    if (Out2) store_node<STREAM>(Out2 + row, r);
                     if (j < g) *reinterpret_cast<P *>(dst + (size_t)threadIdx.x * PB) = r;
                 }
                 if (j < g) lds_barrier();
@@ -491,8 +496,10 @@ static int build_tree_fused_typed(const void *qp, const void *kp, const void *vp
     if (threads == 512 && key == 3 * 16 + 3) HSA_TREE_LAUNCH(512, 3, 3);        // 8 heads, 8 lanes per row
     else if (threads == 512 && key == 4 * 16 + 4) HSA_TREE_LAUNCH(512, 4, 4);   // 16 heads, 16 lanes per row
     else if (threads == 512 && key == 4 * 16 + 3) HSA_TREE_LAUNCH(512, 4, 3);   // 8 heads, 16 lanes per row
+    else if (threads == 512 && key == 3 * 16 + 4) HSA_TREE_LAUNCH(512, 3, 4);   // 16 heads, 8 lanes per row
     else if (threads == 256 && key == 3 * 16 + 3) HSA_TREE_LAUNCH(256, 3, 3);
     else if (threads == 256 && key == 4 * 16 + 3) HSA_TREE_LAUNCH(256, 4, 3);
+    else if (threads == 256 && key == 3 * 16 + 4) HSA_TREE_LAUNCH(256, 3, 4);
     else if (threads == 512) HSA_TREE_LAUNCH(512, -1, -1);
     else if (threads == 256) HSA_TREE_LAUNCH(256, -1, -1);
     else if (threads == 128) HSA_TREE_LAUNCH(128, -1, -1);

@@ -51,13 +51,9 @@ template <typename P> __device__ __forceinline__ P load_once(const void *p) {
     }
 }
 
-// 16-byte store of a node row piece; WHICH = 0 for the first output, 1 for the second copy.
-// HSA_TREE_NTS bit WHICH selects the streaming hint for that output.
-#ifndef HSA_TREE_NTS
-#define HSA_TREE_NTS 0
-#endif
-template <int WHICH, typename P> __device__ __forceinline__ void store_node(void *p, const P &v) {
-    if constexpr (sizeof(P) == 16 && ((HSA_TREE_NTS >> WHICH) & 1)) {
+// 16-byte store of a node row piece, with the streaming hint if STREAM.
+template <bool STREAM, typename P> __device__ __forceinline__ void store_node(void *p, const P &v) {
+    if constexpr (sizeof(P) == 16 && STREAM) {
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
         __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(p));
     } else {
