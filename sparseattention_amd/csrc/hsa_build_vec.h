@@ -21,7 +21,8 @@ __device__ __forceinline__ void load_vec(const typename T::storage *p, float (&f
     }
 }
 
-template <typename T, int VEC>
+// STREAM: the store carries the streaming hint (the row does not stay in the caches)
+template <typename T, int VEC, bool STREAM = false>
 __device__ __forceinline__ void store_vec(typename T::storage *p, const float (&f)[VEC]) {
     if constexpr (VEC == 1) {
         p[0] = from_float<T>(f[0]);
@@ -31,9 +32,12 @@ __device__ __forceinline__ void store_vec(typename T::storage *p, const float (&
 #pragma unroll
         for (int i = 0; i < VEC; ++i) v.e[i] = from_float<T>(f[i]);
         static_assert(sizeof(P) == 16, "vector path moves 16 bytes per lane");
-        // regular store: the rows are read again by the next launch (a streaming store makes the
-        // tree build itself ~8% faster and the attention kernel after it as much slower)
-        *reinterpret_cast<P *>(p) = v;
+        if constexpr (STREAM) {
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            __builtin_nontemporal_store(__builtin_bit_cast(u4, v), reinterpret_cast<u4 *>(p));
+        } else {
+            *reinterpret_cast<P *>(p) = v;
+        }
     }
 }
 
