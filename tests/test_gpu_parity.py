@@ -385,6 +385,31 @@ def test_build_tree_single_launch(case, dtype, threads, tree_knobs):
     assert (fused.float() - stepwise.float()).abs().max() <= atol
 
 
+def test_build_tree_long_sequence_against_level_by_level():
+    """B1 H16 N65536 D128 bf16, both node copies written (537 MB: the size from which the multi-launch
+    build stores with the streaming hint): every level against the one-level op applied to the
+    tree's own previous level, so that nothing but one level's rounding separates the two."""
+    B, H, N, D = 1, 16, 65536, 128
+    g = torch.Generator(device=DEV).manual_seed(5)
+    mk = lambda rows: torch.randn(B, rows, H, D, generator=g, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    qp, kp, vp = mk(N - 1), mk(N - 1), mk(N - 1)
+    kfull = torch.zeros(B, 2 * N - 1, H, D, dtype=torch.bfloat16, device=DEV)
+    vfull = torch.zeros_like(kfull)
+    kfull[:, :N] = mk(N)
+    vfull[:, :N] = mk(N)
+    sa.build_tree(qp, kp, vp, kfull[:, :N], vfull[:, :N], out=kfull[:, N:], out2=vfull[:, N:])
+    assert torch.equal(kfull[:, N:], vfull[:, N:])
+    kc, vc, off = kfull[:, :N], vfull[:, :N], 0
+    for lvl in range(1, N.bit_length()):
+        P = N >> lvl
+        want = sa.build_parent_nodes(qp[:, off:off + P], kp[:, off:off + P], vp[:, off:off + P], kc, vc)
+        got = kfull[:, N + off:N + off + P]
+        assert (got.float() - want.float()).abs().max() <= 2e-2, "level %d" % lvl
+        kc = vc = got
+        off += P
+    assert off == N - 1
+
+
 def test_build_tree_single_launch_on_concurrent_streams(tree_knobs):
     """Launches on different streams overlap on the GPU and must not share arrival counters:
     four streams each build their own tree several times while the others run."""
