@@ -276,7 +276,9 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
  *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit: head size 32, 64 or 128,
  *                R <= 32; fp32: head size 32 or 64, R <= 16: a query-stationary pass, a
  *                key-stationary pass and a reduction of per-block fp32 partial rows for tree
- *                levels >= 4), else the gather kernels; both are deterministic (no atomics)
+ *                levels >= 4), else the gather kernels; both are deterministic (no atomics).
+ *                Tensors that are not 16-byte aligned run on the gather kernels and need the
+ *                workspace size reported for HSA_ATTN_GATHER.
  */
 #include <stddef.h>
 size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo);

@@ -765,9 +765,21 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
                 "workspace too small (%zu bytes)", workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
     float *ws = (float *)workspace;
-    const bool tile_ok = hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
+    bool tile_ok = hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
     if (algo == HSA_ATTN_TILE && !tile_ok)
         return hsa::fail(HSA_ERR_UNSUPPORTED, "tile backward not available for N=%d D=%d L=%d R=%d dtype=%d", N, D, L, R, dtype);
+    // the tile kernels move 16-byte pieces: tensors that are not aligned to that run on the gather
+    // kernels (whose scalar variant takes any address), given a workspace of their size
+    const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dout | (uintptr_t)dq |
+                           (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)workspace) & 15) == 0;
+    if (tile_ok && algo != HSA_ATTN_GATHER && !aligned) {
+        if (algo == HSA_ATTN_TILE) return hsa::fail(HSA_ERR_INVALID, "tile backward needs 16-byte aligned tensors");
+        const size_t need = hsa::bwd_gather_ws_floats(B, N, H, L, R) * sizeof(float);
+        if (workspace_bytes < need)
+            return hsa::fail(HSA_ERR_INVALID, "tensors are not 16-byte aligned: they run on the gather kernels, which "
+                             "need a workspace of %zu bytes (hsa_attn_bwd_workspace_bytes with HSA_ATTN_GATHER)", need);
+        tile_ok = false;
+    }
     if (tile_ok && algo != HSA_ATTN_GATHER) {
         if (dtype == HSA_F32)
             return hsa::attn_bwd_tile_f32_dispatch(q, k, v, dout, dq, dk, dv, ws, B, N, M, H, D, L, R, causal, st);

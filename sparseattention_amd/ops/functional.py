@@ -299,6 +299,8 @@ def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool, algo: 
     if Q.numel() == 0:
         return dq, dk, dv
     lib = _lib.lib()
+    if algo == "auto" and any(t.data_ptr() % 16 for t in (grad_out, Q, K, V)):
+        algo = "gather"  # the tile kernels move 16-byte pieces
     nbytes = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(Q), _lib.algo_code(algo)))
     ws = torch.empty((max(nbytes, 4) + 3) // 4, device=Q.device, dtype=torch.float32)
     with torch.cuda.device(Q.device):

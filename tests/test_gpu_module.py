@@ -425,3 +425,24 @@ def test_unaligned_views_fall_back_to_the_gather_kernel(dtype):
         assert (out.double().cpu() - want).abs().max() < 1e-5
     else:
         _within(out, want, 2e-2, 1e-2, "unaligned bf16")
+    # the backward takes such tensors too (gather formulation)
+    go = odd(N)
+    qr, kr, vr = (x.double().cpu().requires_grad_(True) for x in (q, k, v))
+    oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"], R).backward(go.double().cpu())
+    from sparseattention_amd.ops import functional as fn
+    dq, dk, dv = fn.attention_backward(go, q, k, v, R, True)
+    tol = 2e-5 if dtype == torch.float32 else 3e-2
+    for got, ref in ((dq, qr.grad), (dk, kr.grad), (dv, vr.grad)):
+        assert (got.double().cpu() - ref).abs().max() <= tol * max(1.0, float(ref.abs().max()))
+    # through the C ABI with the tile workspace only: refused with a message, not a fault
+    from sparseattention_amd import _lib
+    lib = _lib.lib()
+    M, L = 2 * N - 1, N.bit_length() - 1
+    small = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(q), _lib.algo_code("auto")))
+    big = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(q), _lib.algo_code("gather")))
+    if small < big:
+        ws = torch.empty(small // 4 + 1, device=DEV, dtype=torch.float32)
+        rc = lib.hsa_attn_bwd(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(go), _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv),
+                              _lib.ptr(ws), small, B, N, M, H, D, L, R, 1, _lib.dtype_code(q), _lib.algo_code("auto"),
+                              _lib.stream_of(q))
+        assert rc == -22 and b"aligned" in lib.hsa_last_error()
