@@ -41,14 +41,10 @@ struct BwdTileParams {
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 
-// Blocks one wavefront walks.  Key pass: 4 where the query blocks that slide along the strip in
-// operand form (NBW+1 when causal, 2 NBW+1 otherwise) and the next block's rows fit the registers,
-// else 1.  Query pass: 4 in every variant (1 only for sequences whose block count is no multiple
-// of four).
-constexpr int bwd_key_strip(int D, int nbw, bool causal) {
-    return ((causal ? nbw + 1 : 2 * nbw + 1) <= 3 && D <= 64) ? 4 : 1;
-}
-constexpr int BWD_QUERY_STRIP = 4;
+// Blocks one wavefront of either pass walks (1 only for sequences whose block count is no multiple
+// of it): leaf blocks (query pass) or query blocks (key pass) slide along the strip in operand
+// form, NBW+1 of them when causal, 2 NBW+1 otherwise.
+constexpr int BWD_STRIP = 4;  // the reduction kernel and the level-5 pairing assume four: a strip is the 64 leaves under a level-6 node
 // Wavefronts per SIMD the query pass is compiled for: two (256 registers) where that holds its
 // operands without spilling, which a strip with five sliding leaf blocks at D = 64 and every
 // variant at D = 128 do not.

@@ -20,7 +20,7 @@
 namespace hsa {
 
 template <typename T, int D>
-int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sbq, int sbk, hipStream_t st);
+int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb, hipStream_t st);
 
 // ---------------------------------------------------------------- parent build
 template <typename T, int VEC> struct BPack { typename T::storage e[VEC]; };
@@ -685,20 +685,19 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.scale_log2e = 1.4426950408889634f * p.scale;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     const int NB = N / TILE_Q;
-    const int sb = NB % 4 == 0 ? BWD_QUERY_STRIP : 1;                               // query pass
-    const int sbk = NB % 4 == 0 ? bwd_key_strip(D, nbw, causal != 0) : 1;           // key pass
-    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, sbk, st)
-           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, sbk, st)
-                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, sbk, st);
+    const int sb = NB % BWD_STRIP == 0 ? BWD_STRIP : 1;
+    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, st)
+           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
+                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
     if (rc != HSA_OK) return rc;
     // the query pass finished levels 1..4 (1..5 when it walked strips); the root row and the rows
     // past 2N-1 are the reduction's in any case
-    int first = level_offset(N, sb == 4 ? 6 : 5);
+    int first = level_offset(N, sb == BWD_STRIP ? 6 : 5);
     if (first > 2 * N - 2) first = 2 * N - 2;
     const size_t n_fin = (size_t)B * (M - first) * H * D;
     if (n_fin) {
         attn_bwd_tile_reduce_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
-            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, sb == 4 ? 2 : 0);
+            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, sb == BWD_STRIP ? 2 : 0);
         rc = check_launch("attn_bwd_tile_reduce_kernel");
     }
     return rc;
