@@ -75,9 +75,9 @@ struct TileParams {
     float scale_log2e;
 };
 
-// wavefronts per workgroup: 8 (two per SIMD, <= 256 VGPRs each) up to 64 channels,
-// 4 (one per SIMD, <= 512 VGPRs) for 128 channels
-template <int D> constexpr int tile_max_wpb() { return D > 64 ? 4 : 8; }
+// wavefronts per workgroup: 8 (two per SIMD, <= 256 VGPRs each) up to 64 channels and five
+// leaf blocks per query block, 4 (one per SIMD, <= 512 VGPRs) for 128 channels or more leaf blocks
+template <int D, int NKL = 1> constexpr int tile_max_wpb() { return (D > 64 || NKL > 5) ? 4 : 8; }
 
 // SB = query blocks per strip.  The strip loop is fully unrolled so that every load lands
 // in its own (virtual) registers: no loop-carried copies, the compiler's waits then cover
@@ -94,7 +94,7 @@ template <int D> constexpr int tile_max_wpb() { return D > 64 ? 4 : 8; }
 // (the operand slots are free once the MFMA operands have been read) and written out as
 // whole rows.  Needs 2R+1+L <= D*2+16 floats per row to fit.
 template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false>
-__global__ void __launch_bounds__(tile_max_wpb<D>() * 64)
+__global__ void __launch_bounds__((tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>() * 64))
 attn_tile_kernel(TileParams p) {
     using M_ = Mma<T>;
     constexpr int KS = D / 32;                         // 32-channel steps of the QK contraction
@@ -107,7 +107,7 @@ attn_tile_kernel(TileParams p) {
     constexpr int BLK_BYTES = TILE_Q * PITCH;          // one 16-row operand block in LDS
     constexpr int WAVE_LDS = 5 * BLK_BYTES;            // q, k, v, near-tree k, near-tree v
 
-    __shared__ __align__(16) unsigned char smem[tile_max_wpb<D>() * WAVE_LDS];
+    __shared__ __align__(16) unsigned char smem[tile_max_wpb<D, NKL>() * WAVE_LDS];
 
     const int lane = threadIdx.x & 63;
     const int r16 = lane & 15;   // MFMA operand row / result column

@@ -11,6 +11,7 @@ namespace hsa {
 // NBW + 1 leaf blocks; up to 2 (R <= 32) otherwise, where it sees 2 NBW + 1
 constexpr int TILE_MAX_NBW_CAUSAL = 4;
 constexpr int TILE_MAX_NBW = 2;
+constexpr int TILE_MAX_NBW_WIDE = 4;
 
 // Experiment knobs of the tile launch: strip length in query blocks (0 = by problem size),
 // wavefronts per workgroup, XCD remap on/off, alternating strip direction on/off.  Initialised
@@ -58,8 +59,11 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS) return false;
     if (M < 2 * N - 1) return false;
-    if ((R + TILE_Q - 1) / TILE_Q > (causal ? TILE_MAX_NBW_CAUSAL : TILE_MAX_NBW)) return false;
-    return true;
+    const int nbw = (R + TILE_Q - 1) / TILE_Q;
+    if (causal) return nbw <= TILE_MAX_NBW_CAUSAL;
+    // without the causal mask: up to five leaf blocks everywhere, seven or nine (one query block per
+    // wavefront) up to 64 channels and without the weights output
+    return nbw <= TILE_MAX_NBW || (nbw <= TILE_MAX_NBW_WIDE && D <= 64 && !want_weights);
 }
 
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
@@ -81,6 +85,7 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     // four or five leaf blocks per query block: shorter strips keep the operands in registers
     if ((R + TILE_Q - 1) / TILE_Q >= (causal ? 3 : 2) && sb > 2) sb = 2;
     if ((R + TILE_Q - 1) / TILE_Q >= 4 && !knobs.sb) sb = 1;  // longer strips spill at five leaf blocks + halo
+    if (!causal && (R + TILE_Q - 1) / TILE_Q > TILE_MAX_NBW) sb = 1;  // seven or nine leaf blocks: one block per wavefront
     while (sb > NB) sb >>= 1;  // NB is a power of two
     p.NS = NB / sb;
     const long units = (long)B * p.NS * H;

@@ -9,7 +9,8 @@ namespace hsa {
 
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
 static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
-    if (wpb > tile_max_wpb<D>()) wpb = tile_max_wpb<D>();
+    constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
+    if (wpb > MAXW) wpb = MAXW;
     const int nwg = (p.n_units + wpb - 1) / wpb;
     const LaunchEvents ev = take_launch_events();
     if (ev.start && ev.stop)
@@ -22,7 +23,8 @@ static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
 
 template <typename T, int D, int NBW, bool CAUSAL>
 static int tile_launch_weights(const TileParams &p, int wpb, hipStream_t st) {
-    if (wpb > tile_max_wpb<D>()) wpb = tile_max_wpb<D>();
+    constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
+    if (wpb > MAXW) wpb = MAXW;
     const int nwg = (p.n_units + wpb - 1) / wpb;
     attn_tile_kernel<T, D, NBW, CAUSAL, 1, true><<<nwg, wpb * 64, 0, st>>>(p);
     return check_launch("attn_tile_kernel (weights)");
@@ -38,6 +40,14 @@ static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) 
     return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
 }
 
+// seven or nine leaf blocks per query block (window radius 33..64 without the causal mask): one
+// block per wavefront, one wavefront per SIMD, head sizes up to 64
+template <typename T, int D, int NBW>
+static int tile_launch_wide(const TileParams &p, int wpb, hipStream_t st) {
+    if constexpr (D <= 64) return tile_launch_one<T, D, NBW, false, 1>(p, wpb, st);
+    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel at this head size");
+}
+
 #define HSA_TILE_INSTANTIATE(T, D)                                                              \
     template <>                                                                                 \
     int attn_tile_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int sb, int wpb,  \
@@ -49,6 +59,8 @@ static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) 
             case 3: return tile_launch_sb<T, D, 1, true>(p, sb, wpb, st);                       \
             case 4: return tile_launch_sb<T, D, 2, false>(p, sb, wpb, st);                      \
             case 5: return tile_launch_sb<T, D, 2, true>(p, sb, wpb, st);                       \
+            case 6: return tile_launch_wide<T, D, 3>(p, wpb, st);                               \
+            case 8: return tile_launch_wide<T, D, 4>(p, wpb, st);                               \
             case 7: return tile_launch_sb<T, D, 3, true>(p, sb, wpb, st);                       \
             case 9: return tile_launch_sb<T, D, 4, true>(p, sb, wpb, st);                       \
         }                                                                                       \

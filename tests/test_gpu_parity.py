@@ -544,16 +544,19 @@ TILE_CASES = [  # B, N, H, D, R
     (1, 64, 3, 32, 20),
     (1, 1024, 8, 32, 16),
 ]
-# causal only: window radius above 32 (four or five leaf blocks per query block)
-TILE_CASES_WIDE = [(2, 256, 4, 64, 48), (1, 512, 2, 64, 64), (1, 128, 2, 128, 50), (2, 256, 3, 32, 64), (1, 64, 2, 64, 33)]
+# window radius above 32: four or five leaf blocks per query block with the causal mask, seven or
+# nine without it (then up to 64 channels only)
+TILE_CASES_WIDE = [(2, 256, 4, 64, 48), (1, 512, 2, 64, 64), (1, 128, 2, 128, 50), (2, 256, 3, 32, 64), (1, 64, 2, 64, 33),
+                   (1, 1024, 2, 64, 40), (1, 32, 2, 32, 64)]
 
 
 @pytest.mark.parametrize("case", TILE_CASES_WIDE)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("strip", [None, "1", "2"])
-def test_attention_tile_wide_causal_window(case, dtype, strip, tile_knobs):
-    """Causal windows of radius 33..64 stay on the tile kernel; the same radius without the causal
-    mask is refused by it (and served by the gather kernel under the automatic choice)."""
+def test_attention_tile_wide_window(case, dtype, strip, tile_knobs):
+    """Windows of radius 33..64 stay on the tile kernel: with the causal mask at every head size,
+    without it up to 64 channels (128-channel heads are refused by it there and served by the
+    gather kernel under the automatic choice)."""
     B, N, H, D, R = case
     if strip is not None:
         tile_knobs(int(strip), -1, -1, -1)
@@ -564,11 +567,15 @@ def test_attention_tile_wide_causal_window(case, dtype, strip, tile_knobs):
     want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"], R, compute_dtype=torch.float64)
     assert_close(out, want, dtype, "tile, wide causal window")
     tn = sa.build_tree_topology(N, False, device=DEV)
-    with pytest.raises(sa.HsaError):
-        fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
     on = oracle.topology_tables(N, False)
-    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R)
     want = oracle.attention_ref(q, k, v, on["forward_idx"], None, R, compute_dtype=torch.float64)
+    if D <= 64:
+        out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
+        assert_close(out, want, dtype, "tile, wide window, not causal")
+    else:
+        with pytest.raises(sa.HsaError):
+            fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R)
     assert_close(out, want, dtype, "automatic choice, wide window, not causal")
 
 
