@@ -880,6 +880,52 @@ def test_attention_backward_tile_fp32_limits():
     fn.attention_backward(*args)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_attention_backward_random_shapes(seed):
+    """Seeded random shapes through whichever backward kernels the dispatcher picks (tile passes with
+    strips of four or of one block, fp32 tile passes, gather formulation), against autograd through
+    the oracle."""
+    rng = np.random.default_rng(2000 + seed)
+    N = int(2 ** rng.integers(1, 10))
+    D = int(rng.choice([16, 20, 32, 64, 128]))
+    H = int(rng.integers(1, 5))
+    B = int(rng.integers(1, 3))
+    R = int(rng.integers(0, 36))
+    causal = bool(rng.integers(0, 2))
+    dtype = [torch.float32, torch.bfloat16, torch.float16][int(rng.integers(0, 3))]
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=seed)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(seed)).to(dtype)
+    o = oracle.topology_tables(N, causal)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"] if causal else None, R).backward(go.double())
+    dq, dk, dv = fn.attention_backward(go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), R, causal)
+    what = "B%d N%d H%d D%d R%d causal=%s %s" % (B, N, H, D, R, causal, dtype)
+    _grad_close(dq, qr.grad, dtype, "dQ " + what)
+    _grad_close(dk, kr.grad, dtype, "dK " + what)
+    _grad_close(dv, vr.grad, dtype, "dV " + what)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_build_tree_random_shapes(seed, tree_knobs):
+    """Seeded random shapes of the whole-tree build, one launch where possible and level passes, against
+    the oracle."""
+    rng = np.random.default_rng(3000 + seed)
+    N = int(2 ** rng.integers(1, 12))
+    D = int(rng.choice([8, 20, 32, 64, 128]))
+    H = int(rng.choice([1, 2, 3, 4, 8, 16]))
+    B = int(rng.integers(1, 4))
+    dtype = [torch.float32, torch.bfloat16, torch.float16][int(rng.integers(0, 3))]
+    g = torch.Generator().manual_seed(seed)
+    qp, kp, vp = (torch.randn(B, N - 1, H, D, generator=g).to(dtype) for _ in range(3))
+    kl, vl = (torch.randn(B, N, H, D, generator=g).to(dtype) for _ in range(2))
+    want = oracle.build_tree_ref(qp, kp, vp, kl, vl, compute_dtype=torch.float64)
+    dev = [t.to(DEV) for t in (qp, kp, vp, kl, vl)]
+    for mode in (2, 0):
+        tree_knobs(mode, 0 if mode else -1)
+        out = sa.build_tree(*dev)
+        assert_close(out, want, dtype, "B%d N%d H%d D%d %s mode %d" % (B, N, H, D, dtype, mode))
+
+
 def test_attention_backward_rejects_unknown_tables():
     N = 16
     q, k, v = make_qkv(1, N, 1, 16, torch.float32, seed=1, M=40)
