@@ -203,9 +203,10 @@ int hsa_build_tree_fwd(const void *qp, const void *kp, const void *vp, const voi
  *                          head count, N >= 8).
  *                      In the single launch, workgroups finish their own subtrees and the last
  *                      one of each group to arrive continues upwards, counted by arrival
- *                      counters inside the library image (one slice per stream; a launch on a
- *                      capturing stream, or on the 33rd distinct stream, takes the multi-launch
- *                      path).
+ *                      counters inside the library image (one slice per stream, and counters
+ *                      of its own, never handed back, for every launch recorded into a graph;
+ *                      a launch on the 32nd distinct stream, or recorded when those are used up
+ *                      or before any eager call on the device, takes the multi-launch path).
  *   workgroup_threads  64 / 128 / 256 / 512: workgroup size of the single launch, 0 = by
  *                      problem size (default)
  * -1 keeps a value.  Process-wide.  Results do not depend on either.

@@ -358,7 +358,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
 // ---- arrival counters ------------------------------------------------------------------------
 // One slice per (device, stream): launches on one stream run in order, so they can share a slice;
 // launches on different streams may overlap and never do.  Counters wrap to zero on the closing
-// arrival, so a slice is all zero between launches.
+// arrival, so a slice is all zero between launches.  The last slice is not a stream's: launches
+// recorded into a graph take their counters from it, each its own and for good (see below).
 constexpr int TREE_SLICES = 32;
 constexpr int TREE_SLICE_COUNTERS = 1 << 16;
 }  // namespace hsa
@@ -392,11 +393,29 @@ static unsigned *tree_counter_slice(hipStream_t st) {
     for (int i = 0; i < g_tree_owners; ++i)
         if (g_tree_owner[i].dev == dev && g_tree_owner[i].stream == st) { slot = i; break; }
     if (slot < 0) {
-        if (g_tree_owners == TREE_SLICES) return nullptr;
+        if (g_tree_owners == TREE_SLICES - 1) return nullptr;
         slot = g_tree_owners++;
         g_tree_owner[slot] = {dev, st};
     }
     return g_tree_base[dev] + (size_t)slot * TREE_SLICE_COUNTERS;
+}
+
+// Counters of a launch that is being recorded into a graph.  The recorded launch may replay on any
+// stream, next to anything, so it cannot borrow a stream's slice: it gets `need` counters of the
+// last slice that no other launch will ever use (a graph does not run concurrently with itself).
+// They are never handed back; once the slice is used up, and while the array's address on this
+// device is still unknown (resolving a symbol is no call to make during a capture), recorded
+// launches take the path that needs no counters.
+static unsigned g_tree_graph_used[TREE_MAX_DEVICES];
+static unsigned *tree_counters_for_capture(long need) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= TREE_MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(g_tree_mu);
+    if (!g_tree_base[dev]) return nullptr;
+    if ((long)g_tree_graph_used[dev] + need > TREE_SLICE_COUNTERS) return nullptr;
+    unsigned *p = g_tree_base[dev] + (size_t)(TREE_SLICES - 1) * TREE_SLICE_COUNTERS + g_tree_graph_used[dev];
+    g_tree_graph_used[dev] += (unsigned)need;
+    return p;
 }
 
 // compute units of the current device (queried once per device)
@@ -418,9 +437,8 @@ static int ilog2_pow2(int x) {
     return ((1 << l) == x) ? l : -1;
 }
 
-// Launches the one-kernel tree build, or returns HSA_ERR_UNSUPPORTED when the shape, the stream
-// (capturing: a captured launch may later run concurrently with others on any stream) or the
-// counter pool does not allow it.
+// Launches the one-kernel tree build, or returns HSA_ERR_UNSUPPORTED when the shape or the counter
+// pool does not allow it.
 template <typename T>
 static int build_tree_fused_typed(const void *qp, const void *kp, const void *vp, const void *k_leaf,
                                   const void *v_leaf, void *out, void *out2, int B, int N, int H, int D,
@@ -484,8 +502,7 @@ static int build_tree_fused_typed(const void *qp, const void *kp, const void *vp
             (void)hipGetLastError();
             return HSA_ERR_UNSUPPORTED;
         }
-        if (cap != hipStreamCaptureStatusNone) return HSA_ERR_UNSUPPORTED;
-        a.counters = tree_counter_slice(st);
+        a.counters = cap != hipStreamCaptureStatusNone ? tree_counters_for_capture(per_batch * B) : tree_counter_slice(st);
         if (!a.counters) return HSA_ERR_UNSUPPORTED;
     }
     const size_t lds = (size_t)3 * threads * 16;

@@ -37,20 +37,49 @@ def test_step_replays_from_a_hip_graph():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         step()
-    # a launch on a capturing stream builds the tree level group by level group (the one-launch
-    # build keeps per-stream arrival counters, and a captured launch may replay on any stream):
-    # the eager runs it is compared with bit for bit take the same route
+    # the recorded tree build is the one-launch kernel with arrival counters of its own (the eager
+    # warm-up above made the counter array's address known): bit for bit the eager result
+    _replays_equal_eager(graph, step, mk, q, qp, kp, vp, kfull, vfull, out, N)
+    # and the multi-launch build agrees with it to the rounding of one multiply-add
     from sparseattention_amd import _lib
+    nodes = kfull[:, N:].clone()
     assert _lib.lib().hsa_build_tree_tune(0, -1) == 0
     try:
-        _replays_equal_eager(graph, step, mk, q, qp, kp, vp, kfull, vfull, out, N)
+        sa.build_tree(qp, kp, vp, kfull[:, :N], vfull[:, :N], out=kfull[:, N:], out2=vfull[:, N:])
+        torch.cuda.synchronize()
     finally:
         assert _lib.lib().hsa_build_tree_tune(1, -1) == 0
-    # and the one-launch build agrees with it to the rounding of one multiply-add
-    nodes = kfull[:, N:].clone()
-    sa.build_tree(qp, kp, vp, kfull[:, :N], vfull[:, :N], out=kfull[:, N:], out2=vfull[:, N:])
-    torch.cuda.synchronize()
     assert (nodes.float() - kfull[:, N:].float()).abs().max() <= 2e-2
+
+
+def test_two_graphs_with_tree_builds_replay_side_by_side():
+    """Two recorded tree builds have arrival counters of their own: their graphs replay on two
+    streams at the same time, repeatedly, and both keep giving the eager result."""
+    B, N, H, D = 4, 2048, 8, 64
+    data = []
+    for i in range(2):
+        g = torch.Generator().manual_seed(40 + i)
+        data.append([torch.randn(B, rows, H, D, generator=g).to(torch.bfloat16).to(DEV) for rows in (N - 1, N - 1, N - 1, N, N)])
+    want = [sa.build_tree(*d) for d in data]       # eager: also makes the counter array's address known
+    torch.cuda.synchronize()
+    outs = [torch.zeros_like(w) for w in want]
+    graphs = []
+    for i in range(2):
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            sa.build_tree(*data[i], out=outs[i])
+        graphs.append(gr)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(5):
+        for o in outs:
+            o.zero_()
+        torch.cuda.synchronize()
+        for i in range(2):
+            with torch.cuda.stream(streams[i]):
+                graphs[i].replay()
+        torch.cuda.synchronize()
+        for i in range(2):
+            assert torch.equal(outs[i], want[i]), "graph %d, replay %d" % (i, rep)
 
 
 def _replays_equal_eager(graph, step, mk, q, qp, kp, vp, kfull, vfull, out, N):
