@@ -607,9 +607,21 @@ def test_attention_tile_weights_vs_oracle(case, dtype, causal):
     per level; dead slots zero; the sibling leaf's weight split over its two slots) and its
     output, against the oracle; every row of weights sums to one."""
     B, N, H, D, R = case
-    if not causal and R > 32:
-        pytest.skip("the tile kernel takes a window radius above 32 only when causal")
     L = N.bit_length() - 1
+    if not causal and R > 32:
+        # weights for a window radius above 32 come from the tile kernel only with the causal mask:
+        # without it the tile kernel refuses and the automatic choice serves them from the gather kernel
+        q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
+        t = sa.build_tree_topology(N, False, device=DEV)
+        o = oracle.topology_tables(N, False)
+        with pytest.raises(sa.HsaError):
+            fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], None, R, return_weights=True, algo="tile")
+        out, w = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], None, R, return_weights=True)
+        want, want_w = oracle.attention_ref(q, k, v, o["forward_idx"], None, R, compute_dtype=torch.float64,
+                                            return_weights=True)
+        assert_close(out, want, dtype, "automatic choice with weights, wide window")
+        assert (w.double().cpu() - want_w).abs().max() < 2e-2
+        return
     if 2 * R + 1 + L > 2 * D + 16:
         pytest.skip("a row of weights does not fit the wavefront's staging area")
     q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
