@@ -13,8 +13,9 @@
 //    (a few 16-byte LDS reads) and step s contracts channel g*D/4 + s of every lane group.
 //  * O^T[channel, query] = V^T P^T.  The scores' result layout (lane = query, registers = keys
 //    4g+i) is exactly the B operand of step i if that step contracts key 4g+i, so P never moves;
-//    the A operand V^T[channel r16, key 4g+i] is read from the row-major LDS block transposed
-//    (4-byte reads, conflict-free: the four lane groups land in four different bank quarters).
+//    the A operand V^T[channel, key 4g+i] is read from the row-major LDS block transposed; column
+//    r16 of output tile j stands for channel r16*D/16 + j, so a lane's values of one key row are
+//    consecutive floats (one 16-byte read per row).
 // Scores, softmax and accumulation are fp32 throughout; exp2 and the final division are the
 // IEEE-accurate ones (1e-5 bar against the fp64 oracle).
 #include "hsa_common.h"
@@ -27,6 +28,7 @@ namespace hsa {
 namespace {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int TQ = 16;            // queries per block
@@ -186,13 +188,24 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
             dst[4 * t] = x[0]; dst[4 * t + 1] = x[1]; dst[4 * t + 2] = x[2]; dst[4 * t + 3] = x[3];
         }
     };
-    // transposed value operand: dst[j][i] = V[row 4g+i][channel 16j + r16]
+    // transposed value operand: dst[j][i] = V[row 4g+i][channel r16*NJ + j].  Column r16 of output
+    // tile j stands for channel r16*NJ + j, so that a lane's NJ values of one row are consecutive
+    // floats: one 16-byte LDS read per row (two at D = 128) instead of NJ 4-byte ones.
     auto get_cols = [&](int slot, float (&dst)[NJ][4]) {
-        const unsigned char *reg = lds + slot * BLK_BYTES + (4 * g) * PITCH + r16 * 4;
+        const unsigned char *reg = lds + slot * BLK_BYTES + (4 * g) * PITCH + r16 * (NJ * 4);
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
+        for (int i = 0; i < 4; ++i) {
+            if constexpr (NJ == 2) {
+                const f32x2 x = *reinterpret_cast<const f32x2 *>(reg + i * PITCH);
+                dst[0][i] = x[0]; dst[1][i] = x[1];
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) dst[j][i] = *reinterpret_cast<const float *>(reg + i * PITCH + 64 * j);
+                for (int t = 0; t < NJ / 4; ++t) {
+                    const f32x4 x = *reinterpret_cast<const f32x4 *>(reg + i * PITCH + 16 * t);
+                    dst[4 * t][i] = x[0]; dst[4 * t + 1][i] = x[1]; dst[4 * t + 2][i] = x[2]; dst[4 * t + 3][i] = x[3];
+                }
+            }
+        }
     };
 
     struct Stage {
@@ -301,19 +314,45 @@ __global__ void __launch_bounds__(F32_WPB * 64) attn_tile_f32_kernel(TileF32Para
         den += __shfl_xor(den, 16, 64);
         den += __shfl_xor(den, 32, 64);
 
-        // O^T tiles: lane = query r16, rows = channels 16j + 4g + i; back to whole rows through LDS
-        unsigned char *oreg = lds + r16 * PITCH + 16 * g;
+        // O^T tiles: lane = query r16, row 4g+i of tile j = channel (4g+i)*NJ + j; back to whole rows
+        // through LDS
+        unsigned char *oreg = lds + r16 * PITCH + (4 * g) * (NJ * 4);
+        if constexpr (NJ <= 4) {
+            f32x4 o[NJ];
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            f32x4 o = {0.f, 0.f, 0.f, 0.f};
+            for (int j = 0; j < NJ; ++j) {
+                o[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int c = 0; c < NKL; ++c) o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(Vl[c][j][i], sc[c][i], o[j], 0, 0, 0);
+                    o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(Vt[j][i], sc[NKL][i], o[j], 0, 0, 0);
+                    o[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(Vu[j][i], sc[NKL + 1][i], o[j], 0, 0, 0);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-#pragma unroll
-                for (int c = 0; c < NKL; ++c) o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vl[c][j][i], sc[c][i], o, 0, 0, 0);
-                o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vt[j][i], sc[NKL][i], o, 0, 0, 0);
-                o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vu[j][i], sc[NKL + 1][i], o, 0, 0, 0);
+                if constexpr (NJ == 2)
+                    *reinterpret_cast<f32x2 *>(oreg + i * 8) = f32x2{o[0][i] / den, o[1][i] / den};
+                else
+                    *reinterpret_cast<f32x4 *>(oreg + i * 16) =
+                        f32x4{o[0][i] / den, o[1][i] / den, o[2][i] / den, o[3][i] / den};
             }
-            *reinterpret_cast<f32x4 *>(oreg + 64 * j) = f32x4{o[0] / den, o[1] / den, o[2] / den, o[3] / den};
+        } else {
+            // eight tiles: written as they are finished, one float each (holding them all would spill)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                f32x4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                    for (int c = 0; c < NKL; ++c) o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vl[c][j][i], sc[c][i], o, 0, 0, 0);
+                    o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vt[j][i], sc[NKL][i], o, 0, 0, 0);
+                    o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vu[j][i], sc[NKL + 1][i], o, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) *reinterpret_cast<float *>(oreg + (i * NJ + j) * 4) = o[i] / den;
+            }
         }
         {
             const unsigned char *src = lds + lrow * PITCH + 16 * lchk;
