@@ -426,6 +426,10 @@ def main():
         desc = desc.replace("N%d" % N, "N%d" % args.seq_len)
         N = args.seq_len
     causal = not args.noncausal
+    if not causal:
+        desc = desc.replace("causal", "not causal")
+    if args.attention_only:
+        desc = desc.replace(", parents built by the tree kernel", ", span nodes drawn i.i.d.")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = _lib.lib()
