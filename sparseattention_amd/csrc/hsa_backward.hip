@@ -618,29 +618,55 @@ static int attn_bwd_typed(const void *q, const void *k, const void *v, const voi
 }
 
 // ---------------------------------------------------------------- initial span nodes
-template <typename T>
+// One thread per (batch, leaf, VEC channels): VEC = 16 bytes of elements when the channel count and
+// the pointers allow it, else 1.
+template <typename T, int VEC>
 __global__ void span_y_bwd_kernel(const typename T::storage *__restrict__ dY, typename T::storage *__restrict__ dX,
                                   int B, int N, int C, int L) {
+    using S = typename T::storage;
+    struct alignas(sizeof(S) * VEC) Pk { S e[VEC]; };
+    const int CV = C / VEC;
     const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const size_t total = (size_t)B * N * C;
+    const size_t total = (size_t)B * N * CV;
     if (t >= total) return;
-    const int c = (int)(t % C);
-    const int n = (int)((t / C) % N);
-    const int b = (int)(t / ((size_t)C * N));
+    const int c = (int)(t % CV) * VEC;
+    const int n = (int)((t / CV) % N);
+    const int b = (int)(t / ((size_t)CV * N));
     // level l holds N >> l rows; a leaf under an unpaired row contributes to no level above it
     int start = 0;
     for (int l = 1; l <= L; ++l) start += N >> l;
-    const typename T::storage *dy = dY + (size_t)b * start * C + c;
-    float acc = 0.f, w = 1.f;
+    const S *dy = dY + (size_t)b * start * C + c;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    float w = 1.f;
     start = 0;
     for (int l = 1; l <= L; ++l) {
         w *= 0.5f;
         const int rows = N >> l;
         if ((n >> l) >= rows) break;
-        acc = fmaf(w, to_float<T>(dy[(size_t)(start + (n >> l)) * C]), acc);
+        const Pk v = *reinterpret_cast<const Pk *>(dy + (size_t)(start + (n >> l)) * C);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] = fmaf(w, to_float<T>(v.e[e]), acc[e]);
         start += rows;
     }
-    dX[t] = from_float<T>(acc);
+    Pk o;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) o.e[e] = from_float<T>(acc[e]);
+    *reinterpret_cast<Pk *>(dX + ((size_t)b * N + n) * C + c) = o;
+}
+
+template <typename T>
+static int span_y_bwd_launch(const void *dy, void *dx, int B, int N, int C, int L, hipStream_t st) {
+    using S = typename T::storage;
+    constexpr int VEC16 = 16 / (int)sizeof(S);
+    const bool vec = C % VEC16 == 0 && ((((uintptr_t)dy | (uintptr_t)dx)) & 15) == 0;
+    const size_t total = (size_t)B * N * (vec ? C / VEC16 : C);
+    const size_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffffUL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    if (vec) span_y_bwd_kernel<T, VEC16><<<(unsigned)blocks, 256, 0, st>>>((const S *)dy, (S *)dx, B, N, C, L);
+    else span_y_bwd_kernel<T, 1><<<(unsigned)blocks, 256, 0, st>>>((const S *)dy, (S *)dx, B, N, C, L);
+    return check_launch("span_y_bwd_kernel");
 }
 
 // ---------------------------------------------------------------- tile backward dispatch
@@ -852,16 +878,13 @@ int hsa_span_input_y_bwd(const void *dy, void *dx, int B, int N, int C, int dtyp
     HSA_REQUIRE(B >= 1 && C >= 1, "bad shape B=%d C=%d", B, C);
     HSA_REQUIRE(N >= 2 && N <= (1 << 26), "N must lie in [2, 2^26] (got %d)", N);
     const int L = hsa::span_levels(N);
-    const size_t total = (size_t)B * N * C;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
-        case HSA_F32: hsa::span_y_bwd_kernel<hsa::F32><<<blocks, 256, 0, st>>>((const float *)dy, (float *)dx, B, N, C, L); break;
-        case HSA_F16: hsa::span_y_bwd_kernel<hsa::F16><<<blocks, 256, 0, st>>>((const uint16_t *)dy, (uint16_t *)dx, B, N, C, L); break;
-        case HSA_BF16: hsa::span_y_bwd_kernel<hsa::BF16><<<blocks, 256, 0, st>>>((const uint16_t *)dy, (uint16_t *)dx, B, N, C, L); break;
-        default: return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+        case HSA_F32: return hsa::span_y_bwd_launch<hsa::F32>(dy, dx, B, N, C, L, st);
+        case HSA_F16: return hsa::span_y_bwd_launch<hsa::F16>(dy, dx, B, N, C, L, st);
+        case HSA_BF16: return hsa::span_y_bwd_launch<hsa::BF16>(dy, dx, B, N, C, L, st);
     }
-    return hsa::check_launch("span_y_bwd_kernel");
+    return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
 }
 
 }  // extern "C"

@@ -965,9 +965,10 @@ def test_build_parents_backward_vs_oracle_autograd(shape, dtype):
 
 
 @pytest.mark.parametrize("N", [64, 100, 37, 3])
+@pytest.mark.parametrize("C", [24, 7, 512])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_span_input_y_backward(dtype, N):
-    B, C = 2, 24
+def test_span_input_y_backward(dtype, N, C):
+    B = 2
     x = torch.randn(B, N, C, generator=torch.Generator().manual_seed(0)).to(dtype)
     gy = torch.randn(B, N - bin(N).count("1"), C, generator=torch.Generator().manual_seed(1)).to(dtype)
     xr = x.double().requires_grad_(True)
