@@ -38,6 +38,8 @@ int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb
             case 3: return bwd_tile_launch_one<T, D, 1, true>(p, sb, st);                        \
             case 4: return bwd_tile_launch_one<T, D, 2, false>(p, sb, st);                       \
             case 5: return bwd_tile_launch_one<T, D, 2, true>(p, sb, st);                        \
+            case 7: return bwd_tile_launch_one<T, D, 3, true>(p, sb, st);                        \
+            case 9: return bwd_tile_launch_one<T, D, 4, true>(p, sb, st);                        \
         }                                                                                        \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward");       \
     }

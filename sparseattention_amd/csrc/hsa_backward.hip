@@ -675,13 +675,20 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
                                void *dv, float *ws, int B, int N, int M, int H, int D, int L, int R, int causal,
                                hipStream_t st);
 
-static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype) {
+// causal: 1 / 0, or -1 when the caller does not know yet (the workspace query): then "eligible
+// with the causal mask only" counts as eligible.  16-bit types take R <= 32, and R <= 64 with the
+// causal mask (at most five leaf blocks per query block either way).
+static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype, int causal) {
     if (dtype == HSA_F32) return attn_bwd_tile_f32_eligible(N, M, D, L, R);
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
-    if ((R + TILE_Q - 1) / TILE_Q > 2) return false;
-    return true;
+    const int nbw = (R + TILE_Q - 1) / TILE_Q;
+    return nbw <= 2 || (nbw <= 4 && causal != 0);
+}
+// the tile passes run only with the causal mask at this radius (16-bit types)
+static bool attn_bwd_tile_needs_causal(int R, int dtype) {
+    return dtype != HSA_F32 && (R + TILE_Q - 1) / TILE_Q > 2;
 }
 
 static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
@@ -772,8 +779,12 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
 }
 
 size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo) {
-    const bool tile = algo != HSA_ATTN_GATHER && hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
-    const size_t fl = tile ? hsa::bwd_tile_ws_floats(B, N, H, D, L) : hsa::bwd_gather_ws_floats(B, N, H, L, R);
+    const bool tile = algo != HSA_ATTN_GATHER && hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype, -1);
+    const size_t tile_fl = hsa::bwd_tile_ws_floats(B, N, H, D, L), gather_fl = hsa::bwd_gather_ws_floats(B, N, H, L, R);
+    size_t fl = tile ? tile_fl : gather_fl;
+    // the query does not say whether the call will be causal: where that decides between the two
+    // formulations, the automatic choice needs room for either
+    if (tile && algo == HSA_ATTN_AUTO && hsa::attn_bwd_tile_needs_causal(R, dtype) && gather_fl > fl) fl = gather_fl;
     return fl * sizeof(float);
 }
 
@@ -790,9 +801,9 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
                 "workspace too small (%zu bytes)", workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
     float *ws = (float *)workspace;
-    bool tile_ok = hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype);
+    bool tile_ok = hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype, causal ? 1 : 0);
     if (algo == HSA_ATTN_TILE && !tile_ok)
-        return hsa::fail(HSA_ERR_UNSUPPORTED, "tile backward not available for N=%d D=%d L=%d R=%d dtype=%d", N, D, L, R, dtype);
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "tile backward not available for N=%d D=%d L=%d R=%d causal=%d dtype=%d", N, D, L, R, causal ? 1 : 0, dtype);
     // the tile kernels move 16-byte pieces: tensors that are not aligned to that run on the gather
     // kernels (whose scalar variant takes any address), given a workspace of their size
     const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)dout | (uintptr_t)dq |

@@ -831,7 +831,10 @@ def _grad_close(got, want, dtype, what):
                                   (2, 256, 3, 64, 32, 600), (1, 1024, 2, 64, 0, None), (1, 64, 12, 64, 9, None),
                                   (1, 128, 2, 128, 32, None), (2, 32, 3, 128, 7, None), (2, 256, 4, 32, 16, None),
                                   (1, 128, 8, 32, 32, None), (1, 2048, 2, 64, 16, None), (1, 512, 3, 32, 20, None),
-                                  (2, 4096, 1, 64, 8, None)])
+                                  (2, 4096, 1, 64, 8, None),
+                                  # window radius 33..64: tile passes with the causal mask, gather formulation without
+                                  (1, 256, 2, 64, 48, None), (2, 128, 3, 32, 64, None), (1, 128, 2, 128, 40, None),
+                                  (1, 1024, 4, 64, 64, None)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
@@ -936,6 +939,26 @@ def test_build_tree_random_shapes(seed, tree_knobs):
         tree_knobs(mode, 0 if mode else -1)
         out = sa.build_tree(*dev)
         assert_close(out, want, dtype, "B%d N%d H%d D%d %s mode %d" % (B, N, H, D, dtype, mode))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_backward_wide_causal_window_on_the_tile_passes(dtype):
+    """Window radius 33..64: the tile passes take it with the causal mask (and agree with the gather
+    formulation), refuse it without, and the automatic choice serves both."""
+    B, N, H, D, R = 2, 512, 4, 64, 56
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=77)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(8)).to(dtype)
+    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), R)
+    tile = fn.attention_backward(*args, True, algo="tile")
+    gath = fn.attention_backward(*args, True, algo="gather")
+    for a, b in zip(tile, gath):
+        assert (a.float() - b.float()).abs().max() <= 4e-2 * max(1.0, float(b.float().abs().max()))
+    with pytest.raises(sa.HsaError):
+        fn.attention_backward(*args, False, algo="tile")
+    auto = fn.attention_backward(*args, False)
+    gath = fn.attention_backward(*args, False, algo="gather")
+    for a, b in zip(auto, gath):
+        assert torch.equal(a, b)
 
 
 def test_attention_backward_rejects_unknown_tables():
