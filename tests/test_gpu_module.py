@@ -59,6 +59,45 @@ def test_lm_at_benchmark_width_vs_oracle(dtype):
     assert e_kernel <= 3 * e_torch + 1e-3, "kernel path error %.3e vs torch 16-bit error %.3e" % (e_kernel, e_torch)
 
 
+@pytest.mark.parametrize("fused", [True, False])
+def test_lm_training_step_gradients_vs_oracle(fused):
+    """One training step of a small decoder LM in fp32 (the reference's whole-model check compares
+    forward and parameter gradients of two models with the same weights,
+    triton_kernel/Hierarchical_Attention_Triton_Forward_Test.py:2088-2282): cross-entropy loss and the
+    gradient of every parameter against autograd through the fp64 oracle, with the span-node update
+    as one differentiable function and level by level."""
+    V, d, H, ff, layers, N, B, R = 101, 64, 4, 128, 2, 64, 2, 5
+    torch.manual_seed(3)
+    m = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation="relu", max_len=N).train()
+    for layer in m.layers:
+        layer.self_attn.fused_training = fused
+    tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(4))
+    tgt = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(5))
+    sd = {k: (v.detach().double().cpu().requires_grad_(v.is_floating_point() and k != "pos_encoding.pe")
+              if v.is_floating_point() else v.cpu()) for k, v in m.state_dict().items()}
+    if "fc_out.weight" in sd:
+        sd["fc_out.weight"] = sd["embedding.weight"]           # tied
+    ref_logits = oracle.lm_forward_ref(sd, tok, H, layers, R, "relu")
+    ref_loss = torch.nn.functional.cross_entropy(ref_logits.view(-1, V), tgt.view(-1))
+    ref_loss.backward()
+    md = m.to(DEV)
+    loss = torch.nn.functional.cross_entropy(md(tok.to(DEV)).view(-1, V), tgt.to(DEV).view(-1))
+    loss.backward()
+    assert abs(loss.item() - ref_loss.item()) < 1e-4
+    checked = 0
+    for name, p in md.named_parameters():
+        ref = sd[name].grad
+        if ref is None:
+            # a parameter the forward never reads (kept for state-dict compatibility): unused on both sides
+            assert p.grad is None or not p.grad.any(), name
+            continue
+        assert p.grad is not None, name
+        err = float((p.grad.double().cpu() - ref).abs().max())
+        assert err <= 2e-5 * max(1.0, float(ref.abs().max())) + 1e-6, "%s: %.3e" % (name, err)
+        checked += 1
+    assert checked >= 10 * layers
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_module_at_benchmark_width_vs_oracle(causal):
     """The module alone at dim 512 / 8 heads / 4096 leaves, bf16 (one layer of the decoder-LM
