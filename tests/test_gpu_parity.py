@@ -961,6 +961,31 @@ def test_attention_backward_wide_causal_window_on_the_tile_passes(dtype):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_backward_long_sequence_upper_levels(causal):
+    """65536 leaves, 16 levels: a node near the root collects its gradient from tens of thousands
+    of queries (the reference keeps a repro script for the magnitude of exactly these gradients,
+    triton_kernel/reproduce_issue_v2.py).  The tile passes (per-strip partial rows summed by the
+    reduction kernel) against the per-key gather formulation, level by level."""
+    B, N, H, D, R = 1, 65536, 2, 64, 16
+    g = torch.Generator(device=DEV).manual_seed(9)
+    mk = lambda rows: torch.randn(B, rows, H, D, generator=g, device=DEV).to(torch.bfloat16)
+    q, k, v, go = mk(N), mk(2 * N - 1), mk(2 * N - 1), mk(N)
+    tile = fn.attention_backward(go, q, k, v, R, causal, algo="tile")
+    gath = fn.attention_backward(go, q, k, v, R, causal, algo="gather")
+    off = N
+    for lvl in range(1, N.bit_length()):
+        rows = N >> lvl
+        for a, b, name in ((tile[1], gath[1], "dK"), (tile[2], gath[2], "dV")):
+            x, y = a[:, off:off + rows].float(), b[:, off:off + rows].float()
+            scale = max(1.0, float(y.abs().max()))
+            assert (x - y).abs().max() <= 3e-2 * scale, "%s level %d (scale %.1f)" % (name, lvl, scale)
+        off += rows
+    assert (tile[0].float() - gath[0].float()).abs().max() <= 3e-2 * max(1.0, float(gath[0].float().abs().max()))
+    # the root row is attended by nobody
+    assert not tile[1][:, 2 * N - 2].any() and not tile[2][:, 2 * N - 2].any()
+
+
 def test_attention_backward_rejects_unknown_tables():
     N = 16
     q, k, v = make_qkv(1, N, 1, 16, torch.float32, seed=1, M=40)
