@@ -14,11 +14,11 @@ constexpr int TILE_MAX_NBW = 2;
 constexpr int TILE_MAX_NBW_WIDE = 4;
 
 // Experiment knobs of the tile launch: strip length in query blocks (0 = by problem size),
-// wavefronts per workgroup, XCD remap on/off, alternating strip direction on/off.  Initialised
+// wavefronts per workgroup (0 = by head count), XCD remap on/off, alternating strip direction on/off.  Initialised
 // once per process from HSA_ATTN_TILE_SB / _WPB / _SWZ / _ALT, changed afterwards only through
 // hsa_attn_tile_tune; a launch reads four atomics, never the environment.
 struct TileKnobs {
-    std::atomic<int> sb{0}, wpb{8}, swizzle{1}, alternate{1};
+    std::atomic<int> sb{0}, wpb{0}, swizzle{1}, alternate{1};
     TileKnobs() {
         if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
         if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) swizzle = atoi(e) != 0;
@@ -39,7 +39,7 @@ void attn_tile_knobs_sb_swizzle(int *sb, int *swizzle) {
 
 int attn_tile_tune(int sb, int wpb, int swizzle, int alternate) {
     if (!(sb == -1 || sb == 0 || sb == 1 || sb == 2 || sb == 4)) return fail(HSA_ERR_INVALID, "strip length %d", sb);
-    if (!(wpb == -1 || (wpb >= 1 && wpb <= 8))) return fail(HSA_ERR_INVALID, "wavefronts per workgroup %d", wpb);
+    if (!(wpb == -1 || (wpb >= 0 && wpb <= 8))) return fail(HSA_ERR_INVALID, "wavefronts per workgroup %d", wpb);
     TileKnobs &k = tile_knobs();
     if (sb >= 0) k.sb = sb;
     if (wpb >= 0) k.wpb = wpb;
@@ -94,7 +94,18 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     p.xcd_swizzle = knobs.swizzle;
     p.alternate = knobs.alternate;
     p.scale_log2e = 1.4426950408889634f / sqrtf((float)D);
-    const int wpb = knobs.wpb;
+    // wavefronts per workgroup: as many as the variant allows, but a divisor of the head count
+    // where one at least half that large exists, so that a workgroup's wavefronts are heads of one
+    // strip and read whole contiguous token rows together (12 heads: 6 per workgroup, 35 -> 32 us
+    // at B8 N2048 D64)
+    int wpb = knobs.wpb;
+    if (wpb == 0) {
+        const int maxw = D > 64 ? 4 : 8;
+        wpb = maxw;
+        if (H % maxw != 0)
+            for (int d = maxw - 1; d >= maxw / 2; --d)
+                if (H % d == 0) { wpb = d; break; }
+    }
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (weights) {
         // one query block per wavefront

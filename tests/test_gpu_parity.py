@@ -41,7 +41,7 @@ def tile_knobs():
     def set_knobs(sb, wpb, swizzle, alternate):
         assert _lib.lib().hsa_attn_tile_tune(sb, wpb, swizzle, alternate) == 0
     yield set_knobs
-    assert _lib.lib().hsa_attn_tile_tune(0, 8, 1, 1) == 0
+    assert _lib.lib().hsa_attn_tile_tune(0, 0, 1, 1) == 0
 
 
 def make_qkv(B, N, H, D, dtype, seed=0, scale=1.0, M=None):
