@@ -105,6 +105,8 @@ __device__ __forceinline__ VPack<T, VEC> combine(const VPack<T, VEC> &q, const V
 // LGG / LGH: log2 of the lanes per head row and of the head count when known at compile time
 // (-1: taken from the arguments).  With both fixed, the subtrees per workgroup, every slot
 // index and the cross-lane sums become constants: about half the instructions per level.
+struct VPackBits { uint32_t x, y, z, w; };
+
 template <typename T, int VEC, int TL, int THREADS, int LGG, int LGH>
 __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
     using S = typename T::storage;
@@ -190,6 +192,27 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
         bk[j - 1] = load_once<P>(Kp + row);
         bv[j - 1] = load_once<P>(Vp + row);
     }
+    // The parent rows of the levels above the workgroups' own (phase C) are read by whichever
+    // workgroup closes a group, right after its arrival and on the critical path of the launch's
+    // tail.  The workgroups of a batch element share them out and touch them now, last in the
+    // request order and with regular loads, so that the closing workgroup finds them in the caches.
+    P touch;
+    {
+        const int first_lvl = TL + lgS + 1;
+        const long rows_top = (long)(N >> (first_lvl - 1)) - 1;   // nodes of levels first_lvl .. root
+        const long ppr = (long)(rs / VEC);                        // 16-byte pieces per row
+        const long n_pieces = rows_top > 0 ? 3 * rows_top * ppr : 1;
+        long t = (long)wg * THREADS + (long)threadIdx.x;
+        if (t >= n_pieces) t = n_pieces - 1;
+        const long per = rows_top > 0 ? rows_top * ppr : 1;
+        const int which = (int)(t / per);
+        const long rem = t - (long)which * per;
+        const S *base = which == 0 ? (const S *)a.qp + (size_t)b * a.qp_bs
+                      : which == 1 ? (const S *)a.kp + (size_t)b * a.kp_bs
+                                   : (const S *)a.vp + (size_t)b * a.vp_bs;
+        const size_t first_row = rows_top > 0 ? (size_t)(level_offset(N, first_lvl) - N) : 0;
+        touch = *reinterpret_cast<const P *>(base + first_row * rs + (size_t)rem * VEC);
+    }
     __builtin_amdgcn_sched_barrier(0);
 
     {
@@ -262,6 +285,8 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
             if (j < lgS) lds_barrier();
         }
     }
+
+    asm volatile("" ::"v"(__builtin_bit_cast(VPackBits, touch).x));
 
     // ---- phase C: the last workgroup of a group to arrive continues upwards ----------------
     int level = TL + lgS;    // this workgroup holds node `idx` of that level (all heads)
