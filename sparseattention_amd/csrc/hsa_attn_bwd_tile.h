@@ -37,6 +37,8 @@ struct BwdTileParams {
     int B, N, M, H, L, R;
     int n_units;
     float scale_log2e, scale;
+    // rows the key pass's trailing workgroups finish from the partial rows (none: red_wgs == 0)
+    int causal, red_first_row, red_wgs;
 };
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
@@ -507,12 +509,20 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     }
 }
 
+template <typename T>
+__device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
+                                                typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D,
+                                                int L, int causal, int first_row, int lg_sb, size_t t);
+
 // ---------------------------------------------------------------------------------------------
 // (B) key-stationary pass over the leaf key blocks
 // ---------------------------------------------------------------------------------------------
 // A wavefront walks SB consecutive key blocks; the query blocks whose window reaches a key block
 // (NQB of them) slide along in registers in operand form, so each query / dO row is fetched once
 // per strip instead of once per key block it touches.
+// The last red_wgs workgroups of the grid do not take key blocks: they sum the query pass's
+// partial rows into the upper tree levels' dK / dV rows (independent of the leaf rows this pass
+// writes), which fills the chip while the key blocks' last loads and stores drain.
 template <typename T, int D, int NBW, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(BWD_WPB * 64)
 attn_bwd_tile_key_kernel(BwdTileParams p) {
@@ -524,6 +534,14 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
     constexpr int LDS_SLOTS = 4;
     __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
 
+    const int key_wgs = (int)gridDim.x - p.red_wgs;
+    if ((int)blockIdx.x >= key_wgs) {
+        using S = typename T::storage;
+        bwd_reduce_rows<T>(p.partial, reinterpret_cast<S *>(p.dk), reinterpret_cast<S *>(p.dv), p.B, p.N, p.M, p.H, D,
+                           p.L, p.causal, p.red_first_row, SB == BWD_STRIP ? 2 : 0,
+                           (size_t)((int)blockIdx.x - key_wgs) * (BWD_WPB * 64) + threadIdx.x);
+        return;
+    }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = blockIdx.x * BWD_WPB + wave;
     if (unit >= p.n_units) return;
@@ -671,22 +689,24 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
 
 // Rows from first_row on (a level the query pass left unfinished, up to anything above row 2N-2):
 // node (l, p) sums the partial rows of the query blocks (levels 4, 5) or strips (levels >= 6)
-// under its sibling; nodes nobody attends (the
-// root, right-hand nodes when causal, rows past 2N-1) get zeros.  One thread per (batch, row,
-// head, channel).  lg_sb = log2 of the blocks per strip of the query pass.
+// under its sibling; nodes nobody attends (the root, right-hand nodes when causal, rows past
+// 2N-1) get zeros.  One thread per (batch, row, head, four channels), index t.  lg_sb = log2 of
+// the blocks per strip of the query pass.
 template <typename T>
-__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
-                                            typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D, int L,
-                                            int causal, int first_row, int lg_sb) {
-    const size_t per_b = (size_t)(M - first_row) * H * D;
-    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
+                                                typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D,
+                                                int L, int causal, int first_row, int lg_sb, size_t t) {
+    using S = typename T::storage;
+    struct alignas(4 * sizeof(S)) Pack { S e[4]; };
+    const int D4 = D / 4;
+    const size_t per_b = (size_t)(M - first_row) * H * D4;
     if (t >= (size_t)B * per_b) return;
     const int b = (int)(t / per_b);
     const size_t r = t % per_b;
-    const int row = first_row + (int)(r / ((size_t)H * D));
-    const int h = (int)((r / D) % H);
-    const int d = (int)(r % D);
-    float vk = 0.f, vv = 0.f;
+    const int row = first_row + (int)(r / ((size_t)H * D4));
+    const int h = (int)((r / D4) % H);
+    const int d = 4 * (int)(r % D4);
+    f32x4 vk = {0.f, 0.f, 0.f, 0.f}, vv = {0.f, 0.f, 0.f, 0.f};
     if (row < 2 * N - 2) {
         int lvl = 4;
         while (row >= level_offset(N, lvl + 1)) ++lvl;
@@ -710,24 +730,38 @@ __global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, t
                 pk = far + (((size_t)b * NS + (blk0 >> lg_sb)) * H + h) * LF * D + (size_t)(lvl - 6) * D + d;
                 pv = pk + (size_t)B * NS * H * LF * D;
             }
-            // eight independent loads in flight per round trip
+            // eight independent 16-byte loads per tensor in flight per round trip
             int i = 0;
             for (; i + 8 <= n; i += 8) {
-                float a[8], c[8];
+                f32x4 a[8], c[8];
 #pragma unroll
-                for (int u = 0; u < 8; ++u) { a[u] = pk[(size_t)(i + u) * stride]; c[u] = pv[(size_t)(i + u) * stride]; }
+                for (int u = 0; u < 8; ++u) {
+                    a[u] = *reinterpret_cast<const f32x4 *>(pk + (size_t)(i + u) * stride);
+                    c[u] = *reinterpret_cast<const f32x4 *>(pv + (size_t)(i + u) * stride);
+                }
 #pragma unroll
                 for (int u = 0; u < 8; ++u) { vk += a[u]; vv += c[u]; }
             }
             for (; i < n; ++i) {
-                vk += pk[(size_t)i * stride];
-                vv += pv[(size_t)i * stride];
+                vk += *reinterpret_cast<const f32x4 *>(pk + (size_t)i * stride);
+                vv += *reinterpret_cast<const f32x4 *>(pv + (size_t)i * stride);
             }
         }
     }
     const size_t o = ((size_t)b * M + row) * H * D + (size_t)h * D + d;
-    dk[o] = from_float<T>(vk);
-    dv[o] = from_float<T>(vv);
+    Pack ok, ov;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) { ok.e[u] = from_float<T>(vk[u]); ov.e[u] = from_float<T>(vv[u]); }
+    *reinterpret_cast<Pack *>(dk + o) = ok;
+    *reinterpret_cast<Pack *>(dv + o) = ov;
+}
+
+template <typename T>
+__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
+                                            typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D, int L,
+                                            int causal, int first_row, int lg_sb) {
+    bwd_reduce_rows<T>(partial, dk, dv, B, N, M, H, D, L, causal, first_row, lg_sb,
+                       (size_t)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 }  // namespace hsa

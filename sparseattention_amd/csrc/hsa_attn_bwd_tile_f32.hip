@@ -538,7 +538,7 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
     int rc = D == 32 ? launch_d<32>(p, nbw, causal != 0, st) : launch_d<64>(p, nbw, causal != 0, st);
     if (rc != HSA_OK) return rc;
     const int first = level_offset(N, 4);
-    const size_t n_fin = (size_t)B * (M - first) * H * D;
+    const size_t n_fin = (size_t)B * (M - first) * H * (D / 4);  // one thread per four channels
     if (n_fin) {
         attn_bwd_tile_reduce_kernel<F32><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
             p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, 0);

@@ -13,7 +13,7 @@ static int bwd_tile_launch_sb(const BwdTileParams &p, hipStream_t st) {
     attn_bwd_tile_query_kernel<T, D, NBW, CAUSAL, SB><<<nwg, BWD_WPB * 64, 0, st>>>(q);
     int rc = check_launch("attn_bwd_tile_query_kernel");
     if (rc != HSA_OK) return rc;
-    attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL, SB><<<nwg, BWD_WPB * 64, 0, st>>>(q);
+    attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL, SB><<<nwg + q.red_wgs, BWD_WPB * 64, 0, st>>>(q);
     return check_launch("attn_bwd_tile_key_kernel");
 }
 

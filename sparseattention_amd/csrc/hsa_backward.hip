@@ -719,21 +719,20 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     const int NB = N / TILE_Q;
     const int sb = NB % BWD_STRIP == 0 ? BWD_STRIP : 1;
-    int rc = D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, st)
-           : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
-                     : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
-    if (rc != HSA_OK) return rc;
-    // the query pass finished levels 1..4 (1..5 when it walked strips); the root row and the rows
-    // past 2N-1 are the reduction's in any case
+    // The query pass finishes levels 1..4 (1..5 when it walks strips); the rows above them, the
+    // root row and the rows past 2N-1 are summed from its partial rows by the trailing workgroups
+    // of the key pass, one thread per four channels.
     int first = level_offset(N, sb == BWD_STRIP ? 6 : 5);
     if (first > 2 * N - 2) first = 2 * N - 2;
-    const size_t n_fin = (size_t)B * (M - first) * H * D;
-    if (n_fin) {
-        attn_bwd_tile_reduce_kernel<T><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
-            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, sb == BWD_STRIP ? 2 : 0);
-        rc = check_launch("attn_bwd_tile_reduce_kernel");
-    }
-    return rc;
+    const size_t red_threads = (size_t)B * (M - first) * H * (D / 4);
+    const size_t red_wgs = (red_threads + BWD_WPB * 64 - 1) / (BWD_WPB * 64);
+    if (red_wgs > 0x3fffffffUL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.causal = causal != 0;
+    p.red_first_row = first;
+    p.red_wgs = (int)red_wgs;
+    return D == 32 ? attn_bwd_tile_launch_td<T, 32>(p, nbw, causal != 0, sb, st)
+         : D == 64 ? attn_bwd_tile_launch_td<T, 64>(p, nbw, causal != 0, sb, st)
+                   : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
 }
 
 }  // namespace hsa
