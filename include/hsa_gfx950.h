@@ -275,11 +275,12 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
  *   workspace    device memory of at least hsa_attn_bwd_workspace_bytes(...) bytes, provided by
  *                the caller (scratch only: nothing in it has to survive the call)
  *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit: head size 32, 64 or 128,
- *                R <= 32, with the causal mask R <= 64; fp32: head size 32 or 64, R <= 16: a
- *                query-stationary pass, a key-stationary pass and a reduction of fp32 partial
- *                rows for the upper tree levels), else the gather kernels; both are
- *                deterministic (no atomics).  The workspace query does not know whether the call
- *                will be causal: for 32 < R <= 64 it reports what either formulation needs.
+ *                R <= 32, and R <= 64 with the causal mask or up to head size 64; fp32: head size
+ *                32 or 64, R <= 16: a query-stationary pass and a key-stationary pass that also
+ *                sums the first pass's fp32 partial rows for the upper tree levels), else the
+ *                gather kernels; both are deterministic (no atomics).  The workspace query does
+ *                not know whether the call will be causal: for 32 < R <= 64 at head size 128 it
+ *                reports what either formulation needs.
  *                Tensors that are not 16-byte aligned run on the gather kernels and need the
  *                workspace size reported for HSA_ATTN_GATHER.
  */

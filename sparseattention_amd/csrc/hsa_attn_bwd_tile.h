@@ -51,7 +51,7 @@ constexpr int BWD_STRIP = 4;  // the reduction kernel and the level-5 pairing as
 // operands without spilling, which a strip with five sliding leaf blocks at D = 64 and every
 // variant at D = 128 do not.
 constexpr int bwd_query_waves(int D, int nkl, int sb) {
-    return (D <= 32 || (D <= 64 && (nkl <= 3 || sb == 1))) ? 2 : 1;
+    return (nkl <= 5 && (D <= 32 || (D <= 64 && (nkl <= 3 || sb == 1)))) ? 2 : 1;
 }
 
 template <typename T, int D>

@@ -24,6 +24,14 @@ static int bwd_tile_launch_one(const BwdTileParams &p, int sb, hipStream_t st) {
     return bwd_tile_launch_sb<T, D, NBW, CAUSAL, 1>(p, st);
 }
 
+// Windows of 33..64 neighbours to either side without the causal mask (seven or nine leaf blocks
+// per query block): head sizes up to 64 hold that many blocks in registers, one wavefront per SIMD.
+template <typename T, int D, int NBW>
+static int bwd_tile_launch_wide(const BwdTileParams &p, int sb, hipStream_t st) {
+    if constexpr (D <= 64) return bwd_tile_launch_one<T, D, NBW, false>(p, sb, st);
+    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward at this head size");
+}
+
 template <typename T, int D>
 int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb, hipStream_t st);
 
@@ -38,7 +46,9 @@ int attn_bwd_tile_launch_td(const BwdTileParams &p, int nbw, bool causal, int sb
             case 3: return bwd_tile_launch_one<T, D, 1, true>(p, sb, st);                        \
             case 4: return bwd_tile_launch_one<T, D, 2, false>(p, sb, st);                       \
             case 5: return bwd_tile_launch_one<T, D, 2, true>(p, sb, st);                        \
+            case 6: return bwd_tile_launch_wide<T, D, 3>(p, sb, st);                             \
             case 7: return bwd_tile_launch_one<T, D, 3, true>(p, sb, st);                        \
+            case 8: return bwd_tile_launch_wide<T, D, 4>(p, sb, st);                             \
             case 9: return bwd_tile_launch_one<T, D, 4, true>(p, sb, st);                        \
         }                                                                                        \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward");       \

@@ -677,18 +677,18 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
 
 // causal: 1 / 0, or -1 when the caller does not know yet (the workspace query): then "eligible
 // with the causal mask only" counts as eligible.  16-bit types take R <= 32, and R <= 64 with the
-// causal mask (at most five leaf blocks per query block either way).
+// causal mask or with heads of at most 64 channels.
 static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype, int causal) {
     if (dtype == HSA_F32) return attn_bwd_tile_f32_eligible(N, M, D, L, R);
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
-    return nbw <= 2 || (nbw <= 4 && causal != 0);
+    return nbw <= 2 || (nbw <= 4 && (causal != 0 || D <= 64));
 }
-// the tile passes run only with the causal mask at this radius (16-bit types)
-static bool attn_bwd_tile_needs_causal(int R, int dtype) {
-    return dtype != HSA_F32 && (R + TILE_Q - 1) / TILE_Q > 2;
+// the tile passes run only with the causal mask at this radius and head size (16-bit types)
+static bool attn_bwd_tile_needs_causal(int R, int D, int dtype) {
+    return dtype != HSA_F32 && (R + TILE_Q - 1) / TILE_Q > 2 && D > 64;
 }
 
 static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
@@ -783,7 +783,7 @@ size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, in
     size_t fl = tile ? tile_fl : gather_fl;
     // the query does not say whether the call will be causal: where that decides between the two
     // formulations, the automatic choice needs room for either
-    if (tile && algo == HSA_ATTN_AUTO && hsa::attn_bwd_tile_needs_causal(R, dtype) && gather_fl > fl) fl = gather_fl;
+    if (tile && algo == HSA_ATTN_AUTO && hsa::attn_bwd_tile_needs_causal(R, D, dtype) && gather_fl > fl) fl = gather_fl;
     return fl * sizeof(float);
 }
 

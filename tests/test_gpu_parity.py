@@ -943,9 +943,9 @@ def test_build_tree_random_shapes(seed, tree_knobs):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_attention_backward_wide_causal_window_on_the_tile_passes(dtype):
-    """Window radius 33..64: the tile passes take it with the causal mask (and agree with the gather
-    formulation), refuse it without, and the automatic choice serves both."""
-    B, N, H, D, R = 2, 512, 4, 64, 56
+    """Window radius 33..64 at 128 channels per head: the tile passes take it with the causal mask
+    (and agree with the gather formulation), refuse it without, and the automatic choice serves both."""
+    B, N, H, D, R = 2, 512, 2, 128, 56
     q, k, v = make_qkv(B, N, H, D, dtype, seed=77)
     go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(8)).to(dtype)
     args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), R)
@@ -959,6 +959,32 @@ def test_attention_backward_wide_causal_window_on_the_tile_passes(dtype):
     gath = fn.attention_backward(*args, False, algo="gather")
     for a, b in zip(auto, gath):
         assert torch.equal(a, b)
+
+
+WIDE_BWD_CASES = [(2, 512, 4, 64, 56), (1, 256, 2, 64, 33), (2, 128, 3, 32, 64), (1, 1024, 2, 32, 40),
+                  (1, 32, 2, 64, 48), (1, 64, 1, 64, 64), (1, 16, 2, 32, 50), (1, 2048, 2, 64, 64)]
+
+
+@pytest.mark.parametrize("case", WIDE_BWD_CASES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_backward_wide_window_tile_passes(case, causal, dtype):
+    """Window radius 33..64 with heads of at most 64 channels, with and without the causal mask
+    (up to nine leaf blocks per query block; strips of four blocks and of one): the tile passes
+    against autograd through the oracle and against the gather formulation."""
+    B, N, H, D, R = case
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=3 * N + R)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(R)).to(dtype)
+    o = oracle.topology_tables(N, causal)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"] if causal else None, R).backward(go.double())
+    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), R, causal)
+    tile = fn.attention_backward(*args, algo="tile")
+    for name, got, want in zip(("dQ", "dK", "dV"), tile, (qr.grad, kr.grad, vr.grad)):
+        _grad_close(got, want, dtype, name + " wide window, causal=%s" % causal)
+    auto = fn.attention_backward(*args)
+    for a, b in zip(auto, tile):
+        assert torch.equal(a, b), "the automatic choice is the tile passes"
 
 
 @pytest.mark.parametrize("causal", [True, False])
