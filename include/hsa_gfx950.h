@@ -66,9 +66,9 @@ const char *hsa_last_error(void);
  *   causal      used only when idx == NULL
  *   dtype       HSA_F32 / HSA_F16 / HSA_BF16
  *   algo        HSA_ATTN_*.  The MFMA tile kernels take canonical tables (idx == NULL),
- *               16 <= N <= 2^22, R <= 32 (16-bit types: R <= 64 with the causal mask, and
- *               without it up to head size 64), head sizes 32 / 64 / 128, and write weights only
- *               for the 16-bit types; everything else runs on the gather kernel
+ *               16 <= N <= 2^22, R <= 32 (16-bit types: R <= 64), head sizes 32 / 64 / 128, and
+ *               write weights only for the 16-bit types (for 32 < R <= 64 without the causal mask
+ *               only up to head size 64); everything else runs on the gather kernel
  */
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,

@@ -61,9 +61,9 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
     if (M < 2 * N - 1) return false;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (causal) return nbw <= TILE_MAX_NBW_CAUSAL;
-    // without the causal mask: up to five leaf blocks everywhere, seven or nine (one query block per
-    // wavefront) up to 64 channels and without the weights output
-    return nbw <= TILE_MAX_NBW || (nbw <= TILE_MAX_NBW_WIDE && D <= 64 && !want_weights);
+    // without the causal mask: up to five leaf blocks everywhere, seven or nine with one query
+    // block per wavefront (the weights output only up to 64 channels per head)
+    return nbw <= TILE_MAX_NBW || (nbw <= TILE_MAX_NBW_WIDE && (D <= 64 || !want_weights));
 }
 
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,

@@ -41,11 +41,17 @@ static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) 
 }
 
 // seven or nine leaf blocks per query block (window radius 33..64 without the causal mask): one
-// block per wavefront, one wavefront per SIMD, head sizes up to 64
+// block per wavefront, one wavefront per SIMD (at 128 channels per head part of the operands
+// lives in per-lane scratch memory)
 template <typename T, int D, int NBW>
 static int tile_launch_wide(const TileParams &p, int wpb, hipStream_t st) {
-    if constexpr (D <= 64) return tile_launch_one<T, D, NBW, false, 1>(p, wpb, st);
-    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel at this head size");
+    return tile_launch_one<T, D, NBW, false, 1>(p, wpb, st);
+}
+// the same with the weights output, head sizes up to 64
+template <typename T, int D, int NBW>
+static int tile_launch_wide_weights(const TileParams &p, int wpb, hipStream_t st) {
+    if constexpr (D <= 64) return tile_launch_weights<T, D, NBW, false>(p, wpb, st);
+    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel's weights at this head size");
 }
 
 #define HSA_TILE_INSTANTIATE(T, D)                                                              \
@@ -76,6 +82,8 @@ static int tile_launch_wide(const TileParams &p, int wpb, hipStream_t st) {
             case 3: return tile_launch_weights<T, D, 1, true>(p, wpb, st);                      \
             case 4: return tile_launch_weights<T, D, 2, false>(p, wpb, st);                     \
             case 5: return tile_launch_weights<T, D, 2, true>(p, wpb, st);                      \
+            case 6: return tile_launch_wide_weights<T, D, 3>(p, wpb, st);                       \
+            case 8: return tile_launch_wide_weights<T, D, 4>(p, wpb, st);                       \
             case 7: return tile_launch_weights<T, D, 3, true>(p, wpb, st);                      \
             case 9: return tile_launch_weights<T, D, 4, true>(p, wpb, st);                      \
         }                                                                                       \

@@ -545,18 +545,17 @@ TILE_CASES = [  # B, N, H, D, R
     (1, 1024, 8, 32, 16),
 ]
 # window radius above 32: four or five leaf blocks per query block with the causal mask, seven or
-# nine without it (then up to 64 channels only)
+# nine without it
 TILE_CASES_WIDE = [(2, 256, 4, 64, 48), (1, 512, 2, 64, 64), (1, 128, 2, 128, 50), (2, 256, 3, 32, 64), (1, 64, 2, 64, 33),
-                   (1, 1024, 2, 64, 40), (1, 32, 2, 32, 64)]
+                   (1, 1024, 2, 64, 40), (1, 32, 2, 32, 64), (2, 512, 2, 128, 64), (1, 64, 1, 128, 33)]
 
 
 @pytest.mark.parametrize("case", TILE_CASES_WIDE)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("strip", [None, "1", "2"])
 def test_attention_tile_wide_window(case, dtype, strip, tile_knobs):
-    """Windows of radius 33..64 stay on the tile kernel: with the causal mask at every head size,
-    without it up to 64 channels (128-channel heads are refused by it there and served by the
-    gather kernel under the automatic choice)."""
+    """Windows of radius 33..64 stay on the tile kernel, with and without the causal mask, and the
+    automatic choice is the tile kernel."""
     B, N, H, D, R = case
     if strip is not None:
         tile_knobs(int(strip), -1, -1, -1)
@@ -569,14 +568,10 @@ def test_attention_tile_wide_window(case, dtype, strip, tile_knobs):
     tn = sa.build_tree_topology(N, False, device=DEV)
     on = oracle.topology_tables(N, False)
     want = oracle.attention_ref(q, k, v, on["forward_idx"], None, R, compute_dtype=torch.float64)
-    if D <= 64:
-        out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
-        assert_close(out, want, dtype, "tile, wide window, not causal")
-    else:
-        with pytest.raises(sa.HsaError):
-            fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
-    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R)
-    assert_close(out, want, dtype, "automatic choice, wide window, not causal")
+    out = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R, algo="tile")
+    assert_close(out, want, dtype, "tile, wide window, not causal")
+    auto = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), tn["forward_idx"], None, R)
+    assert torch.equal(auto, out), "automatic choice, wide window, not causal"
 
 
 @pytest.mark.parametrize("case", TILE_CASES)
@@ -599,7 +594,7 @@ def test_attention_tile_vs_oracle(case, dtype, causal, strip, tile_knobs):
     assert_close(out, want, dtype, "tile")
 
 
-@pytest.mark.parametrize("case", TILE_CASES + [(1, 256, 2, 64, 48), (1, 64, 2, 32, 24)])
+@pytest.mark.parametrize("case", TILE_CASES + [(1, 256, 2, 64, 48), (1, 64, 2, 32, 24), (1, 128, 2, 128, 40), (2, 512, 2, 64, 64)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
 def test_attention_tile_weights_vs_oracle(case, dtype, causal):
@@ -608,9 +603,10 @@ def test_attention_tile_weights_vs_oracle(case, dtype, causal):
     output, against the oracle; every row of weights sums to one."""
     B, N, H, D, R = case
     L = N.bit_length() - 1
-    if not causal and R > 32:
-        # weights for a window radius above 32 come from the tile kernel only with the causal mask:
-        # without it the tile kernel refuses and the automatic choice serves them from the gather kernel
+    if not causal and R > 32 and D > 64:
+        # weights for a window radius above 32 at 128 channels per head come from the tile kernel only
+        # with the causal mask: without it the tile kernel refuses and the automatic choice serves them
+        # from the gather kernel
         q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
         t = sa.build_tree_topology(N, False, device=DEV)
         o = oracle.topology_tables(N, False)
