@@ -38,7 +38,7 @@ struct BwdTileParams {
     int n_units;
     float scale_log2e, scale;
     // rows the key pass's trailing workgroups finish from the partial rows (none: red_wgs == 0)
-    int causal, red_first_row, red_wgs;
+    int causal, red_first_row, red_wgs, red_lg_sb;  // red_lg_sb: log2 of the query pass's blocks per strip
 };
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
@@ -538,7 +538,7 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
     if ((int)blockIdx.x >= key_wgs) {
         using S = typename T::storage;
         bwd_reduce_rows<T>(p.partial, reinterpret_cast<S *>(p.dk), reinterpret_cast<S *>(p.dv), p.B, p.N, p.M, p.H, D,
-                           p.L, p.causal, p.red_first_row, SB == BWD_STRIP ? 2 : 0,
+                           p.L, p.causal, p.red_first_row, p.red_lg_sb,
                            (size_t)((int)blockIdx.x - key_wgs) * (BWD_WPB * 64) + threadIdx.x);
         return;
     }

@@ -9,10 +9,13 @@ template <typename T, int D, int NBW, bool CAUSAL, int SB>
 static int bwd_tile_launch_sb(const BwdTileParams &p, hipStream_t st) {
     BwdTileParams q = p;
     q.n_units = p.n_units / SB;
+    q.red_lg_sb = SB == BWD_STRIP ? 2 : 0;
     const int nwg = (q.n_units + BWD_WPB - 1) / BWD_WPB;
     attn_bwd_tile_query_kernel<T, D, NBW, CAUSAL, SB><<<nwg, BWD_WPB * 64, 0, st>>>(q);
     int rc = check_launch("attn_bwd_tile_query_kernel");
     if (rc != HSA_OK) return rc;
+    // same strip length for the key blocks (shorter strips re-read more query rows: 54 / 55 us
+    // with two / one block against 52; eight blocks change nothing)
     attn_bwd_tile_key_kernel<T, D, NBW, CAUSAL, SB><<<nwg + q.red_wgs, BWD_WPB * 64, 0, st>>>(q);
     return check_launch("attn_bwd_tile_key_kernel");
 }
