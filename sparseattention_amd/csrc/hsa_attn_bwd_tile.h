@@ -13,8 +13,8 @@
 //      written directly.  A node of level l >= 5 collects from the 2^(l-4) blocks under its
 //      sibling: a wavefront that walks a strip of four blocks finishes level 5 itself and sums
 //      the levels above over its strip; what is left is stored as fp32 partial rows (per strip
-//      and level >= 6, or per block and level >= 5 for strips of one block), and a small
-//      reduction kernel sums each node's contiguous run (deterministic, no atomics).
+//      and level >= 6, or per block and level >= 5 for strips of one block), and pass (B)'s
+//      trailing workgroups sum each node's contiguous run (deterministic, no atomics).
 //  (B) key-stationary, one wavefront per (batch, head, 16-leaf key block): loops over the query
 //      blocks whose window reaches the key block, rebuilds P and dS from the saved statistics
 //      and accumulates dK^T = Q^T . dS, dV^T = dO^T . P in registers.  Every leaf row of dK / dV
@@ -46,7 +46,7 @@ constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 // Blocks one wavefront of either pass walks (1 only for sequences whose block count is no multiple
 // of it): leaf blocks (query pass) or query blocks (key pass) slide along the strip in operand
 // form, NBW+1 of them when causal, 2 NBW+1 otherwise.
-constexpr int BWD_STRIP = 4;  // the reduction kernel and the level-5 pairing assume four: a strip is the 64 leaves under a level-6 node
+constexpr int BWD_STRIP = 4;  // the reduction and the level-5 pairing assume four: a strip is the 64 leaves under a level-6 node
 // Wavefronts per SIMD the query pass is compiled for: two (256 registers) where that holds its
 // operands without spilling, which a strip with five sliding leaf blocks at D = 64 and every
 // variant at D = 128 do not.
@@ -754,14 +754,6 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
     for (int u = 0; u < 4; ++u) { ok.e[u] = from_float<T>(vk[u]); ov.e[u] = from_float<T>(vv[u]); }
     *reinterpret_cast<Pack *>(dk + o) = ok;
     *reinterpret_cast<Pack *>(dv + o) = ov;
-}
-
-template <typename T>
-__global__ void attn_bwd_tile_reduce_kernel(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
-                                            typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D, int L,
-                                            int causal, int first_row, int lg_sb) {
-    bwd_reduce_rows<T>(partial, dk, dv, B, N, M, H, D, L, causal, first_row, lg_sb,
-                       (size_t)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 }  // namespace hsa

@@ -15,7 +15,7 @@
 //  (A) query pass, one wavefront per (batch, head, 16-query block): log-sum-exp and delta of its
 //      queries (saved), dQ, and the rows of dK / dV of the tree nodes: levels 1..3 are attended
 //      only from inside the block and written directly, levels >= 4 leave an fp32 partial row per
-//      block and level that the reduction kernel of the 16-bit backward sums.
+//      block and level; the key pass's trailing workgroups sum them.
 //  (B) key pass, one wavefront per (batch, head, 16-leaf key block): dK / dV of the leaves from
 //      the query blocks whose window reaches the block.
 // Scores, softmax and accumulation are fp32 with the accurate exp2 / log2.
@@ -35,6 +35,8 @@ struct BwdF32Params {
     int B, N, M, H, L, R;
     int n_units;
     float scale_log2e, scale;
+    // rows the key pass's trailing workgroups finish from the partial rows
+    int causal, red_first_row, red_wgs;
 };
 
 template <int D>
@@ -101,7 +103,8 @@ __device__ __forceinline__ int near_slot_level(int sl, int &pl) {
 // (A) query pass
 // ---------------------------------------------------------------------------------------------
 template <int D, int NBW, bool CAUSAL>
-__global__ void __launch_bounds__(F32B_WPB * 64) attn_bwd_f32_query_kernel(BwdF32Params p) {
+__global__ void __launch_bounds__(F32B_WPB * 64) __attribute__((amdgpu_waves_per_eu(2)))
+attn_bwd_f32_query_kernel(BwdF32Params p) {
     using BT = F32Blk<D>;
     constexpr int DS = BT::DS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD;
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
@@ -387,6 +390,14 @@ __global__ void __launch_bounds__(F32B_WPB * 64) attn_bwd_f32_key_kernel(BwdF32P
     constexpr int LDS_SLOTS = 2;
     __shared__ __align__(16) unsigned char smem[F32B_WPB * LDS_SLOTS * BT::BLK_BYTES];
 
+    // the last red_wgs workgroups take no key block: they sum the query pass's partial rows into
+    // the dK / dV rows of tree levels >= 4 (rows this pass does not write)
+    const int key_wgs = (int)gridDim.x - p.red_wgs;
+    if ((int)blockIdx.x >= key_wgs) {
+        bwd_reduce_rows<F32>(p.partial, p.dk, p.dv, p.B, p.N, p.M, p.H, D, p.L, p.causal, p.red_first_row, 0,
+                             (size_t)((int)blockIdx.x - key_wgs) * (F32B_WPB * 64) + threadIdx.x);
+        return;
+    }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = blockIdx.x * F32B_WPB + wave;
     if (unit >= p.n_units) return;
@@ -492,7 +503,7 @@ int launch_both(const BwdF32Params &p, hipStream_t st) {
     attn_bwd_f32_query_kernel<D, NBW, CAUSAL><<<nwg, F32B_WPB * 64, 0, st>>>(p);
     int rc = check_launch("attn_bwd_f32_query_kernel");
     if (rc != HSA_OK) return rc;
-    attn_bwd_f32_key_kernel<D, NBW, CAUSAL><<<nwg, F32B_WPB * 64, 0, st>>>(p);
+    attn_bwd_f32_key_kernel<D, NBW, CAUSAL><<<nwg + p.red_wgs, F32B_WPB * 64, 0, st>>>(p);
     return check_launch("attn_bwd_f32_key_kernel");
 }
 
@@ -535,16 +546,16 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
     p.scale = 1.0f / sqrtf((float)D);
     p.scale_log2e = 1.4426950408889634f * p.scale;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
-    int rc = D == 32 ? launch_d<32>(p, nbw, causal != 0, st) : launch_d<64>(p, nbw, causal != 0, st);
-    if (rc != HSA_OK) return rc;
+    // levels 1..3 are finished by the query pass; everything above, the root row and the rows past
+    // 2N-1 by the key pass's trailing workgroups, one thread per four channels
     const int first = level_offset(N, 4);
-    const size_t n_fin = (size_t)B * (M - first) * H * (D / 4);  // one thread per four channels
-    if (n_fin) {
-        attn_bwd_tile_reduce_kernel<F32><<<(unsigned)((n_fin + 255) / 256), 256, 0, st>>>(
-            p.partial, p.dk, p.dv, B, N, M, H, D, L, causal, first, 0);
-        rc = check_launch("attn_bwd_tile_reduce_kernel");
-    }
-    return rc;
+    const size_t red_threads = (size_t)B * (M - first) * H * (D / 4);
+    const size_t red_wgs = (red_threads + F32B_WPB * 64 - 1) / (F32B_WPB * 64);
+    if (red_wgs > 0x3fffffffUL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.causal = causal != 0;
+    p.red_first_row = first;
+    p.red_wgs = (int)red_wgs;
+    return D == 32 ? launch_d<32>(p, nbw, causal != 0, st) : launch_d<64>(p, nbw, causal != 0, st);
 }
 
 }  // namespace hsa

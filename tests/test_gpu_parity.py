@@ -988,7 +988,7 @@ def test_attention_backward_long_sequence_upper_levels(causal):
     """65536 leaves, 16 levels: a node near the root collects its gradient from tens of thousands
     of queries (the reference keeps a repro script for the magnitude of exactly these gradients,
     triton_kernel/reproduce_issue_v2.py).  The tile passes (per-strip partial rows summed by the
-    reduction kernel) against the per-key gather formulation, level by level."""
+    key pass's trailing workgroups) against the per-key gather formulation, level by level."""
     B, N, H, D, R = 1, 65536, 2, 64, 16
     g = torch.Generator(device=DEV).manual_seed(9)
     mk = lambda rows: torch.randn(B, rows, H, D, generator=g, device=DEV).to(torch.bfloat16)
