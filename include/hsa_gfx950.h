@@ -276,7 +276,7 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
  *                the caller (scratch only: nothing in it has to survive the call)
  *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit: head size 32, 64 or 128,
  *                R <= 32, and R <= 64 with the causal mask or up to head size 64; fp32: head size
- *                32 or 64, R <= 16: a query-stationary pass and a key-stationary pass that also
+ *                32 or 64, R <= 32: a query-stationary pass and a key-stationary pass that also
  *                sums the first pass's fp32 partial rows for the upper tree levels), else the
  *                gather kernels; both are deterministic (no atomics).  The workspace query does
  *                not know whether the call will be causal: for 32 < R <= 64 at head size 128 it

@@ -102,8 +102,13 @@ __device__ __forceinline__ int near_slot_level(int sl, int &pl) {
 // ---------------------------------------------------------------------------------------------
 // (A) query pass
 // ---------------------------------------------------------------------------------------------
+// Wavefronts per SIMD the query pass is compiled for: two (256 registers) up to three leaf blocks
+// per query block, where at most a few words spill; one with five leaf blocks at D = 64.
+constexpr int f32b_query_waves(int D, int nkl) { return (D <= 32 || nkl <= 3) ? 2 : 1; }
+
 template <int D, int NBW, bool CAUSAL>
-__global__ void __launch_bounds__(F32B_WPB * 64) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(F32B_WPB * 64)
+__attribute__((amdgpu_waves_per_eu(f32b_query_waves(D, CAUSAL ? NBW + 1 : 2 * NBW + 1))))
 attn_bwd_f32_query_kernel(BwdF32Params p) {
     using BT = F32Blk<D>;
     constexpr int DS = BT::DS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD;
@@ -514,18 +519,20 @@ int launch_d(const BwdF32Params &p, int nbw, bool causal, hipStream_t st) {
         case 1: return launch_both<D, 0, true>(p, st);
         case 2: return launch_both<D, 1, false>(p, st);
         case 3: return launch_both<D, 1, true>(p, st);
+        case 4: return launch_both<D, 2, false>(p, st);
+        case 5: return launch_both<D, 2, true>(p, st);
     }
     return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the fp32 tile backward");
 }
 
 }  // namespace
 
-// fp32 tensors, head size 32 or 64, canonical tables, R <= 16 (at most three leaf blocks per query
+// fp32 tensors, head size 32 or 64, canonical tables, R <= 32 (at most five leaf blocks per query
 // block: all of a block's rows are in flight at once)
 bool attn_bwd_tile_f32_eligible(int N, int M, int D, int L, int R) {
     if (D != 32 && D != 64) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
-    return R <= TILE_Q;
+    return R <= 2 * TILE_Q;
 }
 
 int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,

@@ -858,7 +858,8 @@ def test_attention_backward_vs_oracle_autograd(case, dtype, causal):
 
 
 F32_BWD_TILE_CASES = [(1, 16, 2, 64, 3), (2, 64, 3, 64, 16), (1, 256, 4, 32, 8), (2, 128, 2, 32, 16), (1, 64, 2, 64, 0),
-                      (1, 1024, 8, 64, 16), (1, 4096, 2, 32, 12), (2, 128, 1, 64, 7)]
+                      (1, 1024, 8, 64, 16), (1, 4096, 2, 32, 12), (2, 128, 1, 64, 7),
+                      (2, 256, 2, 64, 22), (1, 512, 3, 64, 32), (2, 128, 2, 32, 17), (1, 64, 2, 32, 32), (1, 32, 1, 64, 25)]
 
 
 @pytest.mark.parametrize("case", F32_BWD_TILE_CASES)
@@ -885,7 +886,7 @@ def test_attention_backward_tile_fp32_limits():
     """Shapes outside the fp32 tile backward are refused with algo="tile" and run on the gather kernels otherwise."""
     q, k, v = make_qkv(1, 64, 2, 64, torch.float32, seed=2)
     go = torch.randn(1, 64, 2, 64)
-    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), 20, True)
+    args = (go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), 40, True)
     with pytest.raises(_lib.HsaError):
         fn.attention_backward(*args, algo="tile")
     fn.attention_backward(*args)
