@@ -494,6 +494,26 @@ def main():
     attn_bwd_ms = e0.elapsed_time(e1) / K
     del gq, dq_, dk_, dv_, wsp
 
+    # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
+    #     the attention kernel (half read, half written), buffers rotated through 1 GiB like the
+    #     inputs above, K copies between one pair of events ---------------------------------------
+    half = prob.attn_bytes // 2 // 2 * 2
+    ncopy = max(3, -(-(1 << 30) // (2 * half)))
+    csrc = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16).normal_() for _ in range(ncopy)]
+    cdst = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16) for _ in range(ncopy)]
+    with torch.cuda.stream(stream):
+        for i in range(min(K, 2 * ncopy)):
+            cdst[i % ncopy].copy_(csrc[i % ncopy])
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(K):
+            cdst[i % ncopy].copy_(csrc[i % ncopy])
+        e1.record(stream)
+    torch.cuda.synchronize()
+    copy_ms = e0.elapsed_time(e1) / K
+    copy_bytes = 2 * half
+    del csrc, cdst
+
     if args.calibrate_copy:
         n = 64 * 2**20 // 2
         src = [torch.randn(n, device=dev).to(torch.bfloat16) for _ in range(5)]
@@ -540,7 +560,12 @@ def main():
                    "step_frac_of_hbm_peak_two_streams": step_algorithmic / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                    "attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
                    "attn_backward_avg_ms": attn_bwd_ms,
-                   "attn_backward_algorithmic_bytes": E * B * H * D * (2 * N + 2 * M + N + 2 * M)},
+                   "attn_backward_algorithmic_bytes": E * B * H * D * (2 * N + 2 * M + N + 2 * M),
+                   "device_copy_of_the_same_bytes": {
+                       "bytes": copy_bytes, "avg_ms": copy_ms, "GBps": copy_bytes / (copy_ms * 1e-3) / 1e9,
+                       "frac_of_hbm_peak": copy_bytes / (copy_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                       "attention_kernel_vs_copy": copy_ms / attn_avg_ms,
+                       "note": "torch's device-to-device copy of as many bytes as one attention launch moves (half read, half written), buffers rotated through 1 GiB, K copies between one pair of events: what a kernel without arithmetic reaches on this GPU"}},
     }
     if with_tree:
         result["roofline_tree"] = {
