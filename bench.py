@@ -497,22 +497,24 @@ def main():
     # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
     #     the attention kernel (half read, half written), buffers rotated through 1 GiB like the
     #     inputs above, K copies between one pair of events ---------------------------------------
-    half = prob.attn_bytes // 2 // 2 * 2
-    ncopy = max(3, -(-(1 << 30) // (2 * half)))
-    csrc = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16).normal_() for _ in range(ncopy)]
-    cdst = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16) for _ in range(ncopy)]
-    with torch.cuda.stream(stream):
-        for i in range(min(K, 2 * ncopy)):
-            cdst[i % ncopy].copy_(csrc[i % ncopy])
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for i in range(K):
-            cdst[i % ncopy].copy_(csrc[i % ncopy])
-        e1.record(stream)
-    torch.cuda.synchronize()
-    copy_ms = e0.elapsed_time(e1) / K
-    copy_bytes = 2 * half
-    del csrc, cdst
+    def copy_reference(nbytes):
+        half = nbytes // 2 // 2 * 2
+        ncopy = max(3, -(-(1 << 30) // (2 * half)))
+        csrc = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16).normal_() for _ in range(ncopy)]
+        cdst = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16) for _ in range(ncopy)]
+        with torch.cuda.stream(stream):
+            for i in range(min(K, 2 * ncopy)):
+                cdst[i % ncopy].copy_(csrc[i % ncopy])
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for i in range(K):
+                cdst[i % ncopy].copy_(csrc[i % ncopy])
+            e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / K, 2 * half
+
+    copy_ms, copy_bytes = copy_reference(prob.attn_bytes)
+    tree_copy_ms, tree_copy_bytes = copy_reference(prob.tree_bytes) if with_tree else (None, None)
 
     if args.calibrate_copy:
         n = 64 * 2**20 // 2
@@ -573,7 +575,8 @@ def main():
             "achieved": tree_bytes / (tree_b2b_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": tree_bytes / (tree_b2b_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes_per_launch": tree_bytes, "avg_launch_ms": tree_b2b_ms,
-            "timing": "K calls between one pair of events on the launch stream (includes the gaps between launches)"}
+            "timing": "K calls between one pair of events on the launch stream (includes the gaps between launches)",
+            "device_copy_of_the_same_bytes_ms": tree_copy_ms}
         result["detail"]["tree_build_avg_launch_ms"] = tree_b2b_ms
         result["detail"]["tree_algorithmic_bytes"] = tree_bytes
         result["detail"]["tree_GBps"] = tree_bytes / (tree_b2b_ms * 1e-3) / 1e9
