@@ -43,6 +43,13 @@ struct BwdTileParams {
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 
+// Hardware hands consecutive workgroup ids to the 8 XCDs in turn; with this remap workgroups that
+// are consecutive in the returned index run on the same XCD, so neighbouring strips (which share
+// halo rows and upper tree nodes) share an L2.
+__device__ __forceinline__ int bwd_xcd_remap(int wg, int nwg) {
+    return (nwg & 7) == 0 ? (wg & 7) * (nwg >> 3) + (wg >> 3) : wg;
+}
+
 // Blocks one wavefront of either pass walks (1 only for sequences whose block count is no multiple
 // of it): leaf blocks (query pass) or query blocks (key pass) slide along the strip in operand
 // form, NBW+1 of them when causal, 2 NBW+1 otherwise.
@@ -145,7 +152,7 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     __shared__ __align__(16) float carry_mem[SB > 1 ? BWD_WPB * 2 * D : 4];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * BWD_WPB + wave;
+    const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * BWD_WPB + wave;
     if (unit >= p.n_units) return;
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
@@ -543,7 +550,7 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
         return;
     }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * BWD_WPB + wave;
+    const int unit = bwd_xcd_remap((int)blockIdx.x, key_wgs) * BWD_WPB + wave;
     if (unit >= p.n_units) return;
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
