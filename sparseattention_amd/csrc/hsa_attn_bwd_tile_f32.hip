@@ -118,7 +118,7 @@ attn_bwd_f32_query_kernel(BwdF32Params p) {
     __shared__ __align__(16) unsigned char smem[F32B_WPB * LDS_SLOTS * BT::BLK_BYTES];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * F32B_WPB + wave;
+    const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * F32B_WPB + wave;
     if (unit >= p.n_units) return;
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
@@ -404,7 +404,7 @@ __global__ void __launch_bounds__(F32B_WPB * 64) attn_bwd_f32_key_kernel(BwdF32P
         return;
     }
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = blockIdx.x * F32B_WPB + wave;
+    const int unit = bwd_xcd_remap((int)blockIdx.x, key_wgs) * F32B_WPB + wave;
     if (unit >= p.n_units) return;
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
