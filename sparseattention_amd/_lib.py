@@ -115,5 +115,30 @@ def require_gpu(*tensors):
             raise HsaError("this op runs on the GPU only; got a %s tensor" % t.device)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t: torch.Tensor):
+    """The current HIP stream of the tensor's device as a raw handle."""
+    if _raw_stream is not None:
+        return c_void_p(_raw_stream(t.device.index))
     return c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class _SameDevice:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_SAME_DEVICE = _SameDevice()
+
+
+def on_device(t: torch.Tensor):
+    """Context that makes the tensor's device the current one for the launches inside; free when
+    it already is."""
+    if t.device.index == torch.cuda.current_device():
+        return _SAME_DEVICE
+    return torch.cuda.device(t.device)

@@ -94,6 +94,8 @@ class HierarchicalAttention(nn.Module):
             offsets.append(offsets[-1] + s)
         return sizes, offsets
 
+    _DIRECT_PROJECTION_MIN_ELEMENTS = 1 << 20
+
     def _heads(self, t: torch.Tensor) -> torch.Tensor:
         return t.view(t.shape[0], -1, self.num_heads, self.head_dim)
 
@@ -119,10 +121,12 @@ class HierarchicalAttention(nn.Module):
         """Weights of several bias-free projections, cast to `dtype` and stacked along the output
         dimension, so one GEMM computes them all (packed: key / value weights in the operand order
         of the fused upper levels); rebuilt when any of them has been written to or moved."""
-        key = tuple((m.weight.data_ptr(), m.weight._version, m.weight.dtype) for m in layers) + (dtype,)
+        # (the parameter dictionary is read directly: Module.__getattr__ costs a microsecond per use)
+        params = [m._parameters["weight"] for m in layers]
+        key = tuple((w.data_ptr(), w._version, w.dtype) for w in params) + (dtype,)
         hit = self._fused.get(name)
         if hit is None or hit[0] != key:
-            ws = [m.weight.detach().to(dtype) for m in layers]
+            ws = [w.detach().to(dtype) for w in params]
             hit = (key, pack_kv_weights(ws[0], ws[1], self.num_heads) if packed else torch.cat(ws, dim=0))
             self._fused[name] = hit
         return hit[1]
@@ -175,7 +179,7 @@ class HierarchicalAttention(nn.Module):
         top_rows = 0 if keep or not self.fuse_top_levels else _lib.lib().hsa_cross_update_top_rows(H, Dh, code)
         kvs, masks = [], []
         src, off = x, 0
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x):
             for lvl, P in enumerate(self.sizes):
                 if 2 * P <= top_rows:
                     # the remaining levels fit one workgroup per batch: a single launch
@@ -229,7 +233,7 @@ class HierarchicalAttention(nn.Module):
         rs = A(D, 3 * D, 3 * D, 3 * D, 2 * D, 2 * D, 3 * D, 3 * D, 3 * D, 2 * D, 2 * D)
         T3 = (N - 1) * 3 * D
         d_above, dx = None, None
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x):
             for lvl in range(len(self.sizes) - 1, -1, -1):
                 P, off = self.sizes[lvl], self.offsets[lvl]
                 g = dy[:, off:off + P]
@@ -294,9 +298,12 @@ class HierarchicalAttention(nn.Module):
         assert y is not None, "y (parents) cannot be None during top-down update"
         q = self._heads(self.Wq_x(x))
         grad = self._needs_autograd((x, y), (self.Wq_x, self.Wk_x, self.Wv_x))
-        if not grad and not (self.training and self.dropout.p > 0) and y.size(1) == N - 1:
+        if (not grad and not (self.training and self.dropout.p > 0) and y.size(1) == N - 1
+                and B * N * D >= self._DIRECT_PROJECTION_MIN_ELEMENTS):
             # leaves and span nodes are projected straight into their rows of the [B, 2N-1, D]
             # key / value buffers (batched GEMMs with a strided output): no concatenated input.
+            # (Four GEMM launches instead of a copy and two: small inputs, where the launches cost
+            # more host time than the copy costs the GPU, take the other branch.)
             # Everything is brought to the type of q first (under autocast the activations and
             # weights are fp32 while the projections come out in the autocast type; GEMMs with an
             # `out=` are not autocast)

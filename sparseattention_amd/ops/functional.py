@@ -89,7 +89,7 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
     if Q.numel() == 0:  # empty batch: nothing to launch
         return (out, weights) if return_weights else out
     lib = _lib.lib()
-    with torch.cuda.device(Q.device):
+    with _lib.on_device(Q):
         if canon is not None and M >= 2 * N - 1:
             rc = lib.hsa_attn_fwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), None, None, _lib.ptr(out),
                                   _lib.ptr(weights), B, N, M, H, D, L, R, int(canon),
@@ -108,6 +108,8 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
 
 
 def _rows_dense(t: torch.Tensor) -> bool:
+    if t.is_contiguous():
+        return True
     B, rows, H, D = t.shape
     return t.stride(3) == 1 and t.stride(2) == D and (rows == 1 or t.stride(1) == H * D)
 
@@ -144,7 +146,7 @@ def build_parents_forward(Q_p, K_p, V_p, K_c, V_c, return_weights: bool = False,
     weights = torch.empty((B, P, H, 3), device=Q_p.device, dtype=Q_p.dtype) if return_weights else None
     if Q_p.numel() == 0:
         return (out, weights) if return_weights else out
-    with torch.cuda.device(Q_p.device):
+    with _lib.on_device(Q_p):
         rc = _lib.lib().hsa_build_parents_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
             _lib.ptr(weights), B, P, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
@@ -174,7 +176,7 @@ def build_parents_strided(Q_p, K_p, V_p, K_c, V_c, out: torch.Tensor,
         rs[i] = t.stride(1)
         bs[i] = t.stride(0) if B > 1 else t.shape[1] * t.stride(1)
     A = ctypes.c_int64 * 7
-    with torch.cuda.device(Q_p.device):
+    with _lib.on_device(Q_p):
         rc = _lib.lib().hsa_build_parents_strided_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c), _lib.ptr(out),
             _lib.ptr(out2), B, P, H, D, A(*bs), A(*rs), _lib.dtype_code(Q_p), _lib.stream_of(Q_p))
@@ -199,7 +201,7 @@ def pack_kv_weights(w_k: torch.Tensor, w_v: torch.Tensor, num_heads: int) -> tor
     assert w_k.shape == (dim, dim) and w_v.shape == (dim, dim) and w_k.dtype == w_v.dtype
     w_k, w_v = w_k.contiguous(), w_v.contiguous()
     packed = torch.empty(2 * dim * dim, dtype=w_k.dtype, device=w_k.device)
-    with torch.cuda.device(w_k.device):
+    with _lib.on_device(w_k):
         rc = _lib.lib().hsa_cross_update_pack_weights(
             _lib.ptr(w_k), _lib.ptr(w_v), _lib.ptr(packed), num_heads, dim // num_heads,
             _lib.dtype_code(w_k), _lib.stream_of(w_k))
@@ -222,7 +224,7 @@ def cross_update_top(src: torch.Tensor, qkv: torch.Tensor, w_packed: torch.Tenso
     assert qkv.shape == (B, C - 1, 3 * dim) and out.shape == (B, C - 1, dim)
     assert qkv.stride(2) == 1 and out.stride(2) == 1
     assert src.dtype == qkv.dtype == w_packed.dtype == out.dtype, "dtype mismatch"
-    with torch.cuda.device(src.device):
+    with _lib.on_device(src):
         rc = _lib.lib().hsa_cross_update_top_fwd(
             _lib.ptr(src), _lib.ptr(qkv), _lib.ptr(w_packed), _lib.ptr(out), B, C, H, Dh, 0,
             qkv.stride(0) if B > 1 else 0, qkv.stride(1) if C > 2 else 0,
@@ -259,7 +261,7 @@ def build_tree(Q_p, K_p, V_p, K_leaf, V_leaf, out: Optional[torch.Tensor] = None
         if not (t.stride(3) == 1 and t.stride(2) == D and t.stride(1) == H * D):
             ts[i] = t.contiguous()
     Q_p, K_p, V_p, K_leaf, V_leaf = ts
-    with torch.cuda.device(Q_p.device):
+    with _lib.on_device(Q_p):
         rc = _lib.lib().hsa_build_tree_fwd(
             _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_leaf), _lib.ptr(V_leaf), _lib.ptr(out),
             _lib.ptr(out2), B, N, H, D, _batch_stride(Q_p), _batch_stride(K_p), _batch_stride(V_p),
@@ -278,7 +280,7 @@ def build_parents_backward(grad_out, Q_p, K_p, V_p, K_c, V_c):
     dkc, dvc = torch.empty_like(K_c), torch.empty_like(V_c)
     if Q_p.numel() == 0:
         return dq, dkp, dvp, dkc, dvc
-    with torch.cuda.device(Q_p.device):
+    with _lib.on_device(Q_p):
         rc = _lib.lib().hsa_build_parents_bwd(
             _lib.ptr(grad_out), _lib.ptr(Q_p), _lib.ptr(K_p), _lib.ptr(V_p), _lib.ptr(K_c), _lib.ptr(V_c),
             _lib.ptr(dq), _lib.ptr(dkp), _lib.ptr(dvp), _lib.ptr(dkc), _lib.ptr(dvc), B, P, H, D,
@@ -303,7 +305,7 @@ def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool, algo: 
         algo = "gather"  # the tile kernels move 16-byte pieces
     nbytes = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(Q), _lib.algo_code(algo)))
     ws = torch.empty((max(nbytes, 4) + 3) // 4, device=Q.device, dtype=torch.float32)
-    with torch.cuda.device(Q.device):
+    with _lib.on_device(Q):
         rc = lib.hsa_attn_bwd(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(grad_out), _lib.ptr(dq),
                               _lib.ptr(dk), _lib.ptr(dv), _lib.ptr(ws), ws.numel() * 4, B, N, M, H, D,
                               L, R, int(bool(causal)), _lib.dtype_code(Q), _lib.algo_code(algo), _lib.stream_of(Q))

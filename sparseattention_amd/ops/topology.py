@@ -72,7 +72,7 @@ def build_tree_topology(seq_len: int, is_causal: bool = True, device="cuda",
     gat = torch.empty((2 * seq_len - 1, 3), dtype=torch.int32, device=dev)
     lib = _lib.lib()
     if dev.type == "cuda":
-        with torch.cuda.device(idx.device):
+        with _lib.on_device(idx):
             rc = lib.hsa_topology_device(seq_len, int(bool(is_causal)), _lib.ptr(idx), _lib.ptr(msk),
                                          _lib.ptr(gat), _lib.stream_of(idx))
     else:
@@ -93,7 +93,7 @@ class _SpanInputY(torch.autograd.Function):
         B, N, C = x.shape
         x = x.contiguous()
         y = torch.empty((B, N - bin(N).count("1"), C), dtype=x.dtype, device=x.device)
-        with torch.cuda.device(x.device):
+        with _lib.on_device(x):
             rc = _lib.lib().hsa_span_input_y(_lib.ptr(x), _lib.ptr(y), B, N, C, _lib.dtype_code(x),
                                              _lib.stream_of(x))
         _lib.check(rc, "hsa_span_input_y")
@@ -106,7 +106,7 @@ class _SpanInputY(torch.autograd.Function):
         dy = dy.contiguous()
         N = ctx.leaves
         dx = torch.empty((B, N, C), dtype=dy.dtype, device=dy.device)
-        with torch.cuda.device(dy.device):
+        with _lib.on_device(dy):
             rc = _lib.lib().hsa_span_input_y_bwd(_lib.ptr(dy), _lib.ptr(dx), B, N, C, _lib.dtype_code(dy),
                                                  _lib.stream_of(dy))
         _lib.check(rc, "hsa_span_input_y_bwd")

@@ -203,14 +203,18 @@ def test_reference_check_configuration_cross_update_y_gradients():
 # ---------------------------------------------------------------- autocast (the reference evaluates under it)
 @pytest.mark.parametrize("amp", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N", [32, 512])
-def test_module_under_autocast(amp, N):
+@pytest.mark.parametrize("direct", [True, False])
+def test_module_under_autocast(amp, N, direct):
     """fp32 module and fp32 activations inside torch.autocast + no_grad, the way the reference's
     validation loop calls the model (Hierarchical_Transformer_Pretrain.py:607-613): projections
     come out in the autocast type while inputs and weights stay fp32.  N=32 takes the fused upper
-    levels directly from the leaves, N=512 goes through strided levels first."""
+    levels directly from the leaves, N=512 goes through strided levels first.  `direct`: keys and
+    values projected straight into their rows (the branch large inputs take) or from the
+    concatenated input (small inputs)."""
     B, dim, H, R = 2, 128, 2, 4
     torch.manual_seed(4)
     m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=R).to(DEV).eval()
+    m._DIRECT_PROJECTION_MIN_ELEMENTS = 0 if direct else 1 << 40
     g = torch.Generator().manual_seed(5)
     x = torch.randn(B, N, dim, generator=g).clamp(-1, 1)
     y = torch.randn(B, N - 1, dim, generator=g).clamp(-1, 1)
@@ -244,6 +248,22 @@ def test_lm_under_autocast(amp):
     want = oracle.lm_forward_ref(sd, tok, H, layers, R)
     stages = 2 + 2 * layers
     _within(got, want, 2e-2 * stages, 1e-2 * stages, "LM under autocast %s" % amp)
+
+
+def test_update_x_from_y_direct_projection_matches_concatenation():
+    """The no-autograd leaf update projects keys and values either from cat([x, y]) (small inputs)
+    or straight into the rows of the key / value buffers (large inputs): same result."""
+    B, N, dim, H, R = 2, 256, 128, 2, 8
+    torch.manual_seed(11)
+    m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=R).to(DEV).to(torch.bfloat16).eval()
+    x = torch.randn(B, N, dim, device=DEV).bfloat16()
+    y = torch.randn(B, N - 1, dim, device=DEV).bfloat16()
+    outs = []
+    with torch.no_grad():
+        for limit in (0, 1 << 40):
+            m._DIRECT_PROJECTION_MIN_ELEMENTS = limit
+            outs.append(m.update_X_from_Y(x, y, mask=True))
+    assert (outs[0].float() - outs[1].float()).abs().max() <= 2e-2
 
 
 # ---------------------------------------------------------------- partly frozen weights, stale caches
