@@ -374,6 +374,27 @@ def wall_ms_per_step(torch, lib, prob, st_list, K, with_tree):
     return (t1 - t0) * 1e3 / K
 
 
+def copy_reference(torch, stream, K, nbytes):
+    """Average duration (ms) of torch's device-to-device copy that moves `nbytes` in all (half read,
+    half written), buffers rotated through 1 GiB, K copies between one pair of events; and the
+    bytes it moved."""
+    dev = torch.device("cuda", torch.cuda.current_device())
+    half = nbytes // 2 // 2 * 2
+    ncopy = max(3, -(-(1 << 30) // (2 * half)))
+    csrc = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16).normal_() for _ in range(ncopy)]
+    cdst = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16) for _ in range(ncopy)]
+    with torch.cuda.stream(stream):
+        for i in range(min(K, 2 * ncopy)):
+            cdst[i % ncopy].copy_(csrc[i % ncopy])
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(K):
+            cdst[i % ncopy].copy_(csrc[i % ncopy])
+        e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / K, 2 * half
+
+
 def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
     """Kernel times, GB/s and fraction of the HBM peak of one configuration, its one-stream step
     time, and its CPU baseline on a bounded sample."""
@@ -400,7 +421,9 @@ def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
            "tree_GBps": prob.tree_bytes / (tree_ms * 1e-3) / 1e9,
            "tree_frac_of_hbm_peak": prob.tree_bytes / (tree_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
            "single_stream_ms_per_step": step_ms,
-           "single_stream_head_queries_per_s": prob.head_queries / (step_ms * 1e-3)}
+           "single_stream_head_queries_per_s": prob.head_queries / (step_ms * 1e-3),
+           "device_copy_of_attn_bytes_ms": copy_reference(torch, stream, K, prob.attn_bytes)[0],
+           "device_copy_of_tree_bytes_ms": copy_reference(torch, stream, K, prob.tree_bytes)[0]}
     del prob
     torch.cuda.empty_cache()
     if cpu_seconds > 0:
@@ -497,24 +520,8 @@ def main():
     # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
     #     the attention kernel (half read, half written), buffers rotated through 1 GiB like the
     #     inputs above, K copies between one pair of events ---------------------------------------
-    def copy_reference(nbytes):
-        half = nbytes // 2 // 2 * 2
-        ncopy = max(3, -(-(1 << 30) // (2 * half)))
-        csrc = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16).normal_() for _ in range(ncopy)]
-        cdst = [torch.empty(half // 2, device=dev, dtype=torch.bfloat16) for _ in range(ncopy)]
-        with torch.cuda.stream(stream):
-            for i in range(min(K, 2 * ncopy)):
-                cdst[i % ncopy].copy_(csrc[i % ncopy])
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for i in range(K):
-                cdst[i % ncopy].copy_(csrc[i % ncopy])
-            e1.record(stream)
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / K, 2 * half
-
-    copy_ms, copy_bytes = copy_reference(prob.attn_bytes)
-    tree_copy_ms, tree_copy_bytes = copy_reference(prob.tree_bytes) if with_tree else (None, None)
+    copy_ms, copy_bytes = copy_reference(torch, stream, K, prob.attn_bytes)
+    tree_copy_ms = copy_reference(torch, stream, K, prob.tree_bytes)[0] if with_tree else None
 
     if args.calibrate_copy:
         n = 64 * 2**20 // 2
