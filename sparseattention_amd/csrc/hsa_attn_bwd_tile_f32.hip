@@ -18,7 +18,9 @@
 //      block and level; the key pass's trailing workgroups sum them.
 //  (B) key pass, one wavefront per (batch, head, 16-leaf key block): dK / dV of the leaves from
 //      the query blocks whose window reaches the block.
-// Scores, softmax and accumulation are fp32 with the accurate exp2 / log2.
+// Scores, softmax and accumulation are fp32; exp2 is the hardware instruction (1 ulp, arguments
+// <= 0), the log-sum-exp uses the library log2, and P is scaled by one correctly rounded reciprocal
+// per query.
 #include "hsa_attn_bwd_tile.h"
 
 namespace hsa {
@@ -263,17 +265,18 @@ attn_bwd_f32_query_kernel(BwdF32Params p) {
     for (int c = 0; c < NKB; ++c)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            sc[c][i] = exp2f(sc[c][i] - mx);
+            sc[c][i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
             den += sc[c][i];
         }
     den += __shfl_xor(den, 16, 64);
     den += __shfl_xor(den, 32, 64);
+    const float inv = 1.0f / den;  // one correctly rounded reciprocal per query
     float delta = 0.f;
 #pragma unroll
     for (int c = 0; c < NKB; ++c)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            sc[c][i] = sc[c][i] / den;  // P
+            sc[c][i] = sc[c][i] * inv;  // P
             delta = fmaf(sc[c][i], dp[c][i], delta);
         }
     delta += __shfl_xor(delta, 16, 64);
@@ -326,7 +329,7 @@ attn_bwd_f32_query_kernel(BwdF32Params p) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float bias = t == 0 ? b2T[i] : b2U[i];
-            pp[i] = exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
+            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
             ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
         }
         f32x4 tk[NJ], tv[NJ];
@@ -480,7 +483,7 @@ __global__ void __launch_bounds__(F32B_WPB * 64) attn_bwd_f32_key_kernel(BwdF32P
             const bool sib = qb == kb && r16 == (ql ^ 1) && (!CAUSAL || (ql & 1));
             const int cnt = (int)win + (int)sib;
             const float bias = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
-            pp[i] = exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[c][i]);
+            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[c][i]);
             ds[i] = pp[i] * (d[i] - del4[c][i]) * p.scale;
         }
 #pragma unroll
