@@ -110,6 +110,26 @@ class TransformerLM(nn.Module):
                 x, y = layer(x, y, mask=mask)
         return self.fc_out(x)
 
+    def generate(self, src, start_token=2, max_len=50, temperature=1.0):
+        """Samples up to `max_len` tokens after the prompt `src`, one full forward per token, and
+        stops at the end-of-sequence id 3 (Hierarchical_Transformer_Pretrain.py:483-505).  As in the
+        reference every forward needs a power-of-two length, so only prompts whose length stays a
+        power of two while tokens are appended get past the first step."""
+        self.eval()
+        device = next(self.parameters()).device
+        tokens = src.to(device)
+        if tokens.dim() == 1:
+            tokens = tokens.unsqueeze(0)
+        with torch.no_grad():
+            for _ in range(max_len):
+                logits = self.forward(tokens)
+                probs = torch.softmax(logits[:, -1, :] / temperature, dim=-1)
+                nxt = torch.multinomial(probs, 1)
+                tokens = torch.cat([tokens, nxt], dim=1)
+                if nxt.item() == 3:
+                    break
+        return tokens
+
     def load_reference_checkpoint(self, state):
         """Loads a reference checkpoint dict (`{'model_state_dict': ...}` or a bare state dict,
         keys optionally prefixed with `module.`)."""

@@ -266,6 +266,20 @@ def test_update_x_from_y_direct_projection_matches_concatenation():
     assert (outs[0].float() - outs[1].float()).abs().max() <= 2e-2
 
 
+def test_lm_generate_appends_a_sampled_token():
+    """`generate` of the reference LM (Hierarchical_Transformer_Pretrain.py:483-505): one forward
+    per new token, sampled from the last position's distribution."""
+    V, d, H, ff, layers, N = 50, 64, 2, 128, 1, 16
+    torch.manual_seed(3)
+    m = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=4, max_len=64).to(DEV)
+    prompt = torch.randint(4, V, (N,), generator=torch.Generator().manual_seed(1))
+    out = m.generate(prompt, max_len=1)
+    assert out.shape == (1, N + 1) and torch.equal(out[0, :N].cpu(), prompt)
+    assert 0 <= int(out[0, N]) < V and not m.training
+    with pytest.raises(AssertionError):     # 17 tokens: no power of two, as in the reference
+        m.generate(prompt, max_len=2)
+
+
 # ---------------------------------------------------------------- partly frozen weights, stale caches
 def test_partly_frozen_module_still_trains_the_rest():
     """Frozen query weights, trainable key / value weights, inputs without gradient: the module
