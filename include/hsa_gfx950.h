@@ -145,13 +145,19 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
                                   int dtype, void *stream);
 
 /*
- * The last levels of HierarchicalAttention.cross_update_Y in one launch
+ * The last levels of HierarchicalAttention.cross_update_Y in one call
  * (hierarchical_attention/modules/attention.py:119-157: per level the children's
  * Wk_y / Wv_y projections :141-142, build_parent_nodes :145-153, the output feeding the next
  * level :157).  16-bit element types.  Starting from C rows `src` (the output of the level
  * below, or the leaves of a short sequence), every remaining level up to the root is computed
- * on chip: projection by MFMA, rounded to the element type like a separate GEMM's output, then
- * the 3-way softmax per parent and head.
+ * by fused kernels: projection by MFMA, rounded to the element type like a separate GEMM's
+ * output, then the 3-way softmax per parent and head, without the projected keys and values ever
+ * reaching memory.  Two forms with identical results: one launch per level with a wavefront per
+ * (batch element, head), all heads streaming their weights on different CUs at once (the default
+ * where `out` allows 16-byte reads: 16-byte aligned, strides multiples of 8 elements), or a single
+ * launch with one workgroup per batch element that keeps the levels in LDS.
+ * hsa_cross_update_top_tune(1) selects the single launch always, (0) the default, (-1) keeps the
+ * setting; process-wide, initial value from HSA_CROSS_TOP_SINGLE.
  *
  *   src    [B, C, H*Dh]      dense rows; C a power of two, 2 <= C <= hsa_cross_update_top_rows
  *   qkv    parents' q | k | v rows ([.., 3*H*Dh] per row), pointing at the first parent of the
@@ -166,6 +172,7 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
  * (0 = not handled: fp32, or a head size other than 32 / 64 / 128, or H*Dh not a multiple of
  * 128); hsa_cross_update_top_fwd returns HSA_ERR_UNSUPPORTED for such shapes.
  */
+int hsa_cross_update_top_tune(int single_launch);
 int hsa_cross_update_top_rows(int H, int Dh, int dtype);
 int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh,
                                   int dtype, void *stream);

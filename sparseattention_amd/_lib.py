@@ -42,6 +42,8 @@ def _declare(lib):
     lib.hsa_build_parents_fwd.restype = I
     lib.hsa_build_parents_strided_fwd.argtypes = [P] * 7 + [I] * 4 + [P, P, I, P]
     lib.hsa_build_parents_strided_fwd.restype = I
+    lib.hsa_cross_update_top_tune.argtypes = [I]
+    lib.hsa_cross_update_top_tune.restype = I
     lib.hsa_cross_update_top_rows.argtypes = [I, I, I]
     lib.hsa_cross_update_top_rows.restype = I
     lib.hsa_cross_update_pack_weights.argtypes = [P, P, P, I, I, I, P]

@@ -17,6 +17,8 @@
 // LDS buffer, which is the next level's input.
 #include "hsa_mma.h"
 
+#include <stdlib.h>
+
 #include <atomic>
 
 namespace hsa {
@@ -40,23 +42,29 @@ template <typename T> __device__ __forceinline__ float rounded(float x) {
     return to_float<T>(from_float<T>(x));
 }
 
-// One level: C children in `cur` (LDS, 16*RT rows readable), C/2 parents out.  Two passes per
-// head over the level's rows: the key columns give the softmax weights, the value columns the
-// output, so only Dh accumulator columns are live at a time.
-template <typename T, int CT2, int RT>
-__device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int row, const unsigned char *cur,
-                                          unsigned char *nxt, int pitch) {
+// One head of one level: C children (rows of `cur`, `pitch` bytes apart, in LDS or in memory),
+// C/2 parents out.  Two passes over the level's rows: the key columns give the softmax weights,
+// the value columns the output, so only Dh accumulator columns are live at a time.  Row tiles
+// reach past the level's last row when it has fewer than 16*RT children: those lanes re-read the
+// last row, and what they compute belongs to no parent and is dropped.
+// PD = weight k-steps in flight (divides Dm / 32).
+template <typename T, int CT2, int RT, bool TO_LDS, int PD>
+__device__ __forceinline__ void top_level_head(const TopParams &p, int b, int h, int C, int row,
+                                               const unsigned char *cur, unsigned char *nxt, int64_t pitch) {
     using M_ = Mma<T>;
     constexpr int Dh = 16 * CT2;
-    constexpr int PD = CT2 >= 8 ? 2 : 4;    // weight k-steps in flight
     constexpr bool EARLY = RT * CT2 <= 8;   // registers allow the parents' rows to be requested before the projection
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, g = lane >> 4;
     const int Dm = p.Dm, NK = Dm / 32, P = C >> 1;
-    const unsigned char *arow = cur + r16 * pitch + 16 * g;
+    const unsigned char *arow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int r = 16 * rt + r16;
+        arow[rt] = cur + (int64_t)(r < C ? r : C - 1) * pitch + 16 * g;
+    }
 
-    for (int h = wave; h < p.H; h += TOP_WAVES) {
+    {
         // parent e of row tile rt in this lane: 8rt + 2g + e, children = accumulator rows 2e, 2e+1
         const uint16_t *prow[RT][2];
         bool valid[RT][2];
@@ -79,18 +87,27 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
         auto project = [&](int half) {
             // packed weights: [half][head][k-step][column tile][lane][8 elements]
             const uint16_t *wp = p.w + ((size_t)(half * p.H + h) * NK * CT2 * 64 + lane) * 8;
-            const unsigned char *ap = arow;
+            int aofs = 0;
             u32x4_t bq[PD][CT2];
+            // rows that come from memory travel with the weights; rows in LDS are read at use
+            u32x4_t aq[TO_LDS ? 1 : PD][RT];
             auto load_b = [&](int u, int kofs) {
 #pragma unroll
                 for (int ct = 0; ct < CT2; ++ct)
                     bq[u][ct] = *reinterpret_cast<const u32x4_t *>(wp + (kofs * CT2 + ct) * 512);
+                if constexpr (!TO_LDS) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        aq[u][rt] = *reinterpret_cast<const u32x4_t *>(arow[rt] + aofs + 64 * kofs);
+                }
             };
             auto step = [&](int u, bool prefetch) {
                 u32x4_t a[RT];
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    a[rt] = *reinterpret_cast<const u32x4_t *>(ap + 16 * rt * pitch + 64 * u);
+                for (int rt = 0; rt < RT; ++rt) {
+                    if constexpr (TO_LDS) a[rt] = *reinterpret_cast<const u32x4_t *>(arow[rt] + aofs + 64 * u);
+                    else a[rt] = aq[u][rt];
+                }
 #pragma unroll
                 for (int ct = 0; ct < CT2; ++ct)
 #pragma unroll
@@ -109,7 +126,7 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
 #pragma unroll
                 for (int u = 0; u < PD; ++u) step(u, true);
                 wp += PD * CT2 * 512;
-                ap += 64 * PD;
+                aofs += 64 * PD;
             }
 #pragma unroll
             for (int u = 0; u < PD; ++u) step(u, false);
@@ -171,7 +188,7 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 uint16_t *orow = p.out + (size_t)b * p.out_bs + (size_t)(row + prel[rt][e]) * p.out_rs + h * Dh + r16;
-                uint16_t *lrow = reinterpret_cast<uint16_t *>(nxt + prel[rt][e] * pitch) + h * Dh + r16;
+                uint16_t *lrow = TO_LDS ? reinterpret_cast<uint16_t *>(nxt + prel[rt][e] * pitch) + h * Dh + r16 : nullptr;
 #pragma unroll
                 for (int c = 0; c < CT2; ++c) {
                     const float o = wgt[rt][e][0] * to_float<T>(rv[rt][e][c]) +
@@ -180,12 +197,36 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
                     const uint16_t r = from_float<T>(o);
                     if (valid[rt][e]) {
                         orow[16 * c] = r;
-                        lrow[16 * c] = r;
+                        if (TO_LDS) lrow[16 * c] = r;
                     }
                 }
             }
         }
     }
+}
+
+// a workgroup's wavefronts share out the heads of one level whose rows are in LDS
+template <typename T, int CT2, int RT>
+__device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int row, const unsigned char *cur,
+                                          unsigned char *nxt, int pitch) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int PD = CT2 >= 8 ? 2 : 4;  // eight wavefronts per workgroup: 256 registers each
+    for (int h = wave; h < p.H; h += TOP_WAVES) top_level_head<T, CT2, RT, true, PD>(p, b, h, C, row, cur, nxt, pitch);
+}
+
+// One level per launch, one wavefront per (batch element, head): the level's rows are read from
+// memory (the previous launch's output, or the first level's children), so all B*H heads stream
+// their weights on different CUs at once instead of H heads taking turns on one.  The launch
+// boundary is what orders the levels.
+// A lone wavefront per workgroup has 512 registers: PD weight k-steps (PD * Dh/16 KiB) are in
+// flight, which is what bounds a wavefront that streams its head's weights from L2.
+template <typename T, int CT2, int RT, int PD>
+__global__ void __launch_bounds__(64) cross_update_level_kernel(TopParams p, int C, int row, const uint16_t *lsrc,
+                                                                int64_t lsrc_bs, int64_t lsrc_rs) {
+    const int b = blockIdx.x, h = blockIdx.y;
+    top_level_head<T, CT2, RT, false, PD>(p, b, h, C, row,
+                                          reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs), nullptr,
+                                          lsrc_rs * 2);
 }
 
 template <typename T, int CT2, int RT0>
@@ -290,8 +331,49 @@ int top_launch_rt(const TopParams &p, hipStream_t st) {
     return check_launch("cross_update_top_kernel");
 }
 
+// 0 = one launch per level where the result rows allow 16-byte reads, 1 = always the single launch.
+// Initialised once from HSA_CROSS_TOP_SINGLE, changed afterwards through hsa_cross_update_top_tune.
+static std::atomic<int> &top_single_launch() {
+    static std::atomic<int> v{[] { const char *e = getenv("HSA_CROSS_TOP_SINGLE"); return e && atoi(e) != 0 ? 1 : 0; }()};
+    return v;
+}
+
+template <typename T, int CT2, int PD>
+int top_launch_levels_pd(const TopParams &p, hipStream_t st) {
+    const dim3 grid((unsigned)p.B, (unsigned)p.H);
+    int C = p.C0, row = 0;
+    const uint16_t *lsrc = p.src;
+    int64_t lbs = p.src_bs, lrs = p.Dm;
+    while (C >= 2) {
+        if (C >= 64) {
+            if constexpr (CT2 <= 4) cross_update_level_kernel<T, CT2, 4, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+            else return fail(HSA_ERR_UNSUPPORTED, "too many rows (%d) for head_dim %d", C, 16 * CT2);
+        } else if (C >= 32) {
+            cross_update_level_kernel<T, CT2, 2, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+        } else {
+            cross_update_level_kernel<T, CT2, 1, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+        }
+        // the next level's children are the rows just written
+        lsrc = p.out + (size_t)row * p.out_rs;
+        lbs = p.out_bs;
+        lrs = p.out_rs;
+        row += C >> 1;
+        C >>= 1;
+    }
+    return check_launch("cross_update_level_kernel");
+}
+
+template <typename T, int CT2>
+int top_launch_levels(const TopParams &p, hipStream_t st) {
+    constexpr int DEEP = CT2 >= 8 ? 4 : 8;
+    if ((p.Dm / 32) % DEEP == 0) return top_launch_levels_pd<T, CT2, DEEP>(p, st);
+    return top_launch_levels_pd<T, CT2, DEEP / 2>(p, st);
+}
+
 template <typename T, int CT2>
 int top_launch_ct(const TopParams &p, hipStream_t st) {
+    if (!top_single_launch().load() && ((uintptr_t)p.out & 15) == 0 && p.out_rs % 8 == 0 && p.out_bs % 8 == 0)
+        return top_launch_levels<T, CT2>(p, st);
     const int rt0 = p.C0 >= 64 ? 4 : (p.C0 >= 32 ? 2 : 1);
     if constexpr (CT2 <= 4) {
         if (rt0 == 4) return top_launch_rt<T, CT2, 4>(p, st);
@@ -316,6 +398,12 @@ int top_launch(const TopParams &p, int Dh, hipStream_t st) {
 }  // namespace hsa
 
 extern "C" {
+
+int hsa_cross_update_top_tune(int single_launch) {
+    if (single_launch < -1 || single_launch > 1) return hsa::fail(HSA_ERR_INVALID, "single_launch %d", single_launch);
+    if (single_launch >= 0) hsa::top_single_launch().store(single_launch);
+    return HSA_OK;
+}
 
 int hsa_cross_update_top_rows(int H, int Dh, int dtype) {
     if (!hsa::top_shape_ok(H, Dh, dtype)) return 0;

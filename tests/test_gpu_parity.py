@@ -44,6 +44,18 @@ def tile_knobs():
     assert _lib.lib().hsa_attn_tile_tune(0, 0, 1, 1) == 0
 
 
+@pytest.fixture
+def top_knob():
+    """Chooses between one launch per level (0) and the single launch (1) of the span-node update's
+    upper levels for one test and restores the default."""
+    from sparseattention_amd import _lib
+
+    def set_knob(single_launch):
+        assert _lib.lib().hsa_cross_update_top_tune(single_launch) == 0
+    yield set_knob
+    assert _lib.lib().hsa_cross_update_top_tune(0) == 0
+
+
 def make_qkv(B, N, H, D, dtype, seed=0, scale=1.0, M=None):
     g = torch.Generator().manual_seed(seed)
     M = M or 2 * N - 1
@@ -264,9 +276,12 @@ def test_build_parents_column_slices(shape, dtype):
 @pytest.mark.parametrize("B,C,H,Dh", [(2, 64, 8, 64), (3, 32, 4, 32), (1, 2, 2, 64), (2, 16, 2, 128), (2, 32, 4, 128),
                                       (1, 8, 16, 32), (2, 64, 12, 32)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_cross_update_top_levels(B, C, H, Dh, dtype):
-    """All levels above C rows in one launch: against the mathematics in fp64 (projection, 3-way
-    softmax, level after level) and against the level-by-level kernels."""
+@pytest.mark.parametrize("single", [0, 1])
+def test_cross_update_top_levels(B, C, H, Dh, dtype, single, top_knob):
+    """All levels above C rows in one call (one fused launch per level, or a single launch):
+    against the mathematics in fp64 (projection, 3-way softmax, level after level) and against the
+    level-by-level kernels."""
+    top_knob(single)
     dim = H * Dh
     assert C <= fn.fused_top_rows(H, Dh, dtype)
     g = torch.Generator().manual_seed(C + H)
@@ -301,6 +316,27 @@ def test_cross_update_top_levels(B, C, H, Dh, dtype):
         ref.append(cur)
         off, P = off + P, P // 2
     assert (got.float() - torch.cat(ref, dim=1).float()).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("B,C,H,Dh", [(2, 64, 8, 64), (2, 32, 12, 64), (3, 16, 4, 128), (1, 64, 16, 32)])
+def test_cross_update_top_both_forms_agree(B, C, H, Dh, top_knob):
+    """One launch per level and the single launch round at the same places: same bits.  Result rows
+    that do not allow 16-byte reads (odd row stride) take the single launch by themselves."""
+    dim = H * Dh
+    g = torch.Generator().manual_seed(7 * C + H)
+    src = torch.randn(B, C, dim, generator=g).clamp(-1, 1).to(torch.bfloat16).to(DEV)
+    qkv = torch.randn(B, C - 1, 3 * dim, generator=g).clamp(-1, 1).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(2 * dim, dim, generator=g) / dim ** 0.5).to(torch.bfloat16).to(DEV)
+    wp = fn.pack_kv_weights(w[:dim], w[dim:], H)
+    outs = []
+    for single in (0, 1):
+        top_knob(single)
+        outs.append(fn.cross_update_top(src, qkv, wp, torch.empty(B, C - 1, dim, dtype=torch.bfloat16, device=DEV), H))
+    assert torch.equal(outs[0], outs[1])
+    top_knob(0)
+    wide = torch.full((B, C - 1, dim + 4), 3.0, dtype=torch.bfloat16, device=DEV)
+    got = fn.cross_update_top(src, qkv, wp, wide[:, :, :dim], H)
+    assert torch.equal(got, outs[0]) and (wide[:, :, dim:] == 3).all()
 
 
 def test_cross_update_top_shapes_not_handled():
