@@ -159,7 +159,7 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
  * hsa_cross_update_top_tune(1) selects the single launch always, (0) the default, (-1) keeps the
  * setting; process-wide, initial value from HSA_CROSS_TOP_SINGLE.
  *
- *   src    [B, C, H*Dh]      dense rows; C a power of two, 2 <= C <= hsa_cross_update_top_rows
+ *   src    [B, C, H*Dh]      dense rows; C a power of two >= 2 (see hsa_cross_update_top_rows)
  *   qkv    parents' q | k | v rows ([.., 3*H*Dh] per row), pointing at the first parent of the
  *          first level computed here; the C-1 parents follow level after level, root last
  *   w_kv   the Wk_y / Wv_y weights in the kernel's operand order, 2*(H*Dh)^2 elements,
@@ -168,12 +168,17 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
  *   out    result rows, numbered like qkv's, H*Dh elements each
  *   *_bs, *_rs  batch / row strides in elements (0 = dense)
  *
- * hsa_cross_update_top_rows returns the largest C the kernel holds for this head layout
+ * hsa_cross_update_top_rows returns the largest C the single launch holds for this head layout
  * (0 = not handled: fp32, or a head size other than 32 / 64 / 128, or H*Dh not a multiple of
- * 128); hsa_cross_update_top_fwd returns HSA_ERR_UNSUPPORTED for such shapes.
+ * 128); hsa_cross_update_top_fwd returns HSA_ERR_UNSUPPORTED for such shapes, and for a larger C
+ * unless `out` allows the launch per level, which takes any power of two.
+ * hsa_cross_update_level_rows returns the C from which on a caller with such an `out` should hand
+ * the remaining levels to hsa_cross_update_top_fwd instead of running a GEMM and a parent build
+ * per level: at least hsa_cross_update_top_rows, more for small batches (B*C <= 4096).
  */
 int hsa_cross_update_top_tune(int single_launch);
 int hsa_cross_update_top_rows(int H, int Dh, int dtype);
+int hsa_cross_update_level_rows(int B, int H, int Dh, int dtype);
 int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh,
                                   int dtype, void *stream);
 int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv, void *out, int B,

@@ -44,6 +44,8 @@ def _declare(lib):
     lib.hsa_build_parents_strided_fwd.restype = I
     lib.hsa_cross_update_top_tune.argtypes = [I]
     lib.hsa_cross_update_top_tune.restype = I
+    lib.hsa_cross_update_level_rows.argtypes = [I, I, I, I]
+    lib.hsa_cross_update_level_rows.restype = I
     lib.hsa_cross_update_top_rows.argtypes = [I, I, I]
     lib.hsa_cross_update_top_rows.restype = I
     lib.hsa_cross_update_pack_weights.argtypes = [P, P, P, I, I, I, P]

@@ -48,9 +48,14 @@ template <typename T> __device__ __forceinline__ float rounded(float x) {
 // reach past the level's last row when it has fewer than 16*RT children: those lanes re-read the
 // last row, and what they compute belongs to no parent and is dropped.
 // PD = weight k-steps in flight (divides Dm / 32).
+// `tile0`: first 16-row tile of the level this call covers (RT tiles from there).
 template <typename T, int CT2, int RT, bool TO_LDS, int PD>
 __device__ __forceinline__ void top_level_head(const TopParams &p, int b, int h, int C, int row,
-                                               const unsigned char *cur, unsigned char *nxt, int64_t pitch) {
+                                               const unsigned char *cur, unsigned char *nxt, int64_t pitch,
+                                               int tile0 = 0) {
+    // no implicit fusing of multiplies and adds: every instantiation of this function (row tiles
+    // in turn or side by side) rounds at the same places; the fused ones are written as fmaf
+#pragma clang fp contract(off)
     using M_ = Mma<T>;
     constexpr int Dh = 16 * CT2;
     constexpr bool EARLY = RT * CT2 <= 8;   // registers allow the parents' rows to be requested before the projection
@@ -60,7 +65,7 @@ __device__ __forceinline__ void top_level_head(const TopParams &p, int b, int h,
     const unsigned char *arow[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const int r = 16 * rt + r16;
+        const int r = 16 * (tile0 + rt) + r16;
         arow[rt] = cur + (int64_t)(r < C ? r : C - 1) * pitch + 16 * g;
     }
 
@@ -73,7 +78,7 @@ __device__ __forceinline__ void top_level_head(const TopParams &p, int b, int h,
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-                const int pe = 8 * rt + 2 * g + e;
+                const int pe = 8 * (tile0 + rt) + 2 * g + e;
                 valid[rt][e] = pe < P;
                 prel[rt][e] = valid[rt][e] ? pe : P - 1;
                 prow[rt][e] = p.qkv + (size_t)b * p.qkv_bs + (size_t)(row + prel[rt][e]) * p.qkv_rs + h * Dh + r16;
@@ -191,9 +196,10 @@ __device__ __forceinline__ void top_level_head(const TopParams &p, int b, int h,
                 uint16_t *lrow = TO_LDS ? reinterpret_cast<uint16_t *>(nxt + prel[rt][e] * pitch) + h * Dh + r16 : nullptr;
 #pragma unroll
                 for (int c = 0; c < CT2; ++c) {
-                    const float o = wgt[rt][e][0] * to_float<T>(rv[rt][e][c]) +
-                                    wgt[rt][e][1] * rounded<T>(acc[rt][c][2 * e]) +
-                                    wgt[rt][e][2] * rounded<T>(acc[rt][c][2 * e + 1]);
+                    // explicit fused multiply-adds: every instantiation rounds at the same places
+                    const float o = fmaf(wgt[rt][e][2], rounded<T>(acc[rt][c][2 * e + 1]),
+                                         fmaf(wgt[rt][e][1], rounded<T>(acc[rt][c][2 * e]),
+                                              wgt[rt][e][0] * to_float<T>(rv[rt][e][c])));
                     const uint16_t r = from_float<T>(o);
                     if (valid[rt][e]) {
                         orow[16 * c] = r;
@@ -219,14 +225,16 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
 // their weights on different CUs at once instead of H heads taking turns on one.  The launch
 // boundary is what orders the levels.
 // A lone wavefront per workgroup has 512 registers: PD weight k-steps (PD * Dh/16 KiB) are in
-// flight, which is what bounds a wavefront that streams its head's weights from L2.
-template <typename T, int CT2, int RT, int PD>
+// flight, which is what bounds a wavefront that streams its head's weights from L2.  A level of
+// more than 16 children is shared out in 16-row tiles (blockIdx.z), each streaming the weights
+// again: the tiles run side by side instead of one wavefront multiplying them in turn.
+template <typename T, int CT2, int PD>
 __global__ void __launch_bounds__(64) cross_update_level_kernel(TopParams p, int C, int row, const uint16_t *lsrc,
                                                                 int64_t lsrc_bs, int64_t lsrc_rs) {
     const int b = blockIdx.x, h = blockIdx.y;
-    top_level_head<T, CT2, RT, false, PD>(p, b, h, C, row,
-                                          reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs), nullptr,
-                                          lsrc_rs * 2);
+    top_level_head<T, CT2, 1, false, PD>(p, b, h, C, row,
+                                         reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs), nullptr,
+                                         lsrc_rs * 2, (int)blockIdx.z);
 }
 
 template <typename T, int CT2, int RT0>
@@ -338,21 +346,19 @@ static std::atomic<int> &top_single_launch() {
     return v;
 }
 
+// one launch per level reads the previous level's result rows 16 bytes at a time
+static bool top_levels_eligible(const TopParams &p) {
+    return !top_single_launch().load() && ((uintptr_t)p.out & 15) == 0 && p.out_rs % 8 == 0 && p.out_bs % 8 == 0;
+}
+
 template <typename T, int CT2, int PD>
 int top_launch_levels_pd(const TopParams &p, hipStream_t st) {
-    const dim3 grid((unsigned)p.B, (unsigned)p.H);
     int C = p.C0, row = 0;
     const uint16_t *lsrc = p.src;
     int64_t lbs = p.src_bs, lrs = p.Dm;
     while (C >= 2) {
-        if (C >= 64) {
-            if constexpr (CT2 <= 4) cross_update_level_kernel<T, CT2, 4, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
-            else return fail(HSA_ERR_UNSUPPORTED, "too many rows (%d) for head_dim %d", C, 16 * CT2);
-        } else if (C >= 32) {
-            cross_update_level_kernel<T, CT2, 2, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
-        } else {
-            cross_update_level_kernel<T, CT2, 1, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
-        }
+        const dim3 grid((unsigned)p.B, (unsigned)p.H, (unsigned)((C + 15) / 16));
+        cross_update_level_kernel<T, CT2, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
         // the next level's children are the rows just written
         lsrc = p.out + (size_t)row * p.out_rs;
         lbs = p.out_bs;
@@ -372,8 +378,7 @@ int top_launch_levels(const TopParams &p, hipStream_t st) {
 
 template <typename T, int CT2>
 int top_launch_ct(const TopParams &p, hipStream_t st) {
-    if (!top_single_launch().load() && ((uintptr_t)p.out & 15) == 0 && p.out_rs % 8 == 0 && p.out_bs % 8 == 0)
-        return top_launch_levels<T, CT2>(p, st);
+    if (top_levels_eligible(p)) return top_launch_levels<T, CT2>(p, st);
     const int rt0 = p.C0 >= 64 ? 4 : (p.C0 >= 32 ? 2 : 1);
     if constexpr (CT2 <= 4) {
         if (rt0 == 4) return top_launch_rt<T, CT2, 4>(p, st);
@@ -410,6 +415,18 @@ int hsa_cross_update_top_rows(int H, int Dh, int dtype) {
     return 16 * hsa::top_row_tiles(H, Dh);
 }
 
+int hsa_cross_update_level_rows(int B, int H, int Dh, int dtype) {
+    if (B < 1 || !hsa::top_shape_ok(H, Dh, dtype)) return 0;
+    const int held = 16 * hsa::top_row_tiles(H, Dh);
+    if (hsa::top_single_launch().load()) return held;
+    // one launch per level re-reads a head's weights for every 16 rows: it beats a GEMM and a
+    // parent build per level while the batch's rows of a level are few (measured on the LM forward
+    // at 4096 tokens: up to 4096 rows at batch 1, 1024 at 4, 512 at 8, no gain from 32 on)
+    int rows = held;
+    while ((long)B * rows * 2 <= 4096) rows *= 2;
+    return rows;
+}
+
 int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh, int dtype,
                                   void *stream) {
     HSA_REQUIRE(wk && wv && packed, "null pointer");
@@ -431,9 +448,6 @@ int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv,
     HSA_REQUIRE(C >= 2 && hsa::ilog2_exact(C) >= 0, "row count must be a power of two >= 2 (got %d)", C);
     if (!hsa::top_shape_ok(H, Dh, dtype))
         return hsa::fail(HSA_ERR_UNSUPPORTED, "shape H=%d Dh=%d dtype=%d not handled by the fused levels", H, Dh, dtype);
-    if (C > 16 * hsa::top_row_tiles(H, Dh))
-        return hsa::fail(HSA_ERR_UNSUPPORTED, "%d rows exceed the %d the fused levels hold", C,
-                         16 * hsa::top_row_tiles(H, Dh));
     const int64_t Dm = (int64_t)H * Dh;
     if (!src_bs) src_bs = (int64_t)C * Dm;
     if (!qkv_rs) qkv_rs = 3 * Dm;
@@ -451,6 +465,10 @@ int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv,
     p.src_bs = src_bs; p.qkv_bs = qkv_bs; p.qkv_rs = qkv_rs; p.out_bs = out_bs; p.out_rs = out_rs;
     p.B = B; p.H = H; p.Dm = (int)Dm; p.C0 = C;
     p.scale = 1.0f / sqrtf((float)Dh);
+    // the single launch holds a level in registers and LDS; a launch per level takes any size
+    if (C > 16 * hsa::top_row_tiles(H, Dh) && !hsa::top_levels_eligible(p))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "%d rows exceed the %d the single launch holds", C,
+                         16 * hsa::top_row_tiles(H, Dh));
     if (dtype == HSA_BF16) return hsa::top_launch<hsa::BF16>(p, Dh, (hipStream_t)stream);
     return hsa::top_launch<hsa::F16>(p, Dh, (hipStream_t)stream);
 }

@@ -176,13 +176,14 @@ class HierarchicalAttention(nn.Module):
         fwd, code, stream = _lib.lib().hsa_build_parents_strided_fwd, _lib.dtype_code(x), _lib.stream_of(x)
         qkv_p, blk_p, out_p = qkv.data_ptr(), blocks.data_ptr(), y_new.data_ptr()
         # child rows the fused upper levels take (0: shape not handled)
-        top_rows = 0 if keep or not self.fuse_top_levels else _lib.lib().hsa_cross_update_top_rows(H, Dh, code)
+        # (y_new's rows are 16-byte aligned: the fused upper levels may run as a launch per level)
+        top_rows = 0 if keep or not self.fuse_top_levels else _lib.lib().hsa_cross_update_level_rows(B, H, Dh, code)
         kvs, masks = [], []
         src, off = x, 0
         with _lib.on_device(x):
             for lvl, P in enumerate(self.sizes):
                 if 2 * P <= top_rows:
-                    # the remaining levels fit one workgroup per batch: a single launch
+                    # the remaining levels: fused projection + parent build, no GEMM launches
                     w_top = self._fused_weight("kv_y_packed", (self.Wk_y, self.Wv_y), cdt, packed=True)
                     assert src.dtype == cdt and src.is_contiguous() and w_top.dtype == cdt
                     rc = _lib.lib().hsa_cross_update_top_fwd(

@@ -339,7 +339,42 @@ def test_cross_update_top_both_forms_agree(B, C, H, Dh, top_knob):
     assert torch.equal(got, outs[0]) and (wide[:, :, dim:] == 3).all()
 
 
-def test_cross_update_top_shapes_not_handled():
+@pytest.mark.parametrize("B,C,H,Dh", [(1, 1024, 4, 64), (2, 256, 8, 64), (1, 128, 2, 128)])
+def test_cross_update_top_many_rows_per_level_launches(B, C, H, Dh, top_knob):
+    """More children than the single launch holds: one launch per level takes them in 16-row tiles
+    (against the level-by-level kernels); the single launch refuses."""
+    dim = H * Dh
+    assert C > fn.fused_top_rows(H, Dh, torch.bfloat16)
+    g = torch.Generator().manual_seed(C + H)
+    src = torch.randn(B, C, dim, generator=g).clamp(-1, 1).to(torch.bfloat16).to(DEV)
+    qkv = torch.randn(B, C - 1, 3 * dim, generator=g).clamp(-1, 1).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(2 * dim, dim, generator=g) / dim ** 0.5).to(torch.bfloat16).to(DEV)
+    wp = fn.pack_kv_weights(w[:dim], w[dim:], H)
+    got = fn.cross_update_top(src, qkv, wp, torch.empty(B, C - 1, dim, dtype=torch.bfloat16, device=DEV), H)
+    cur, off, P, ref = src, 0, C // 2, []
+    while P >= 1:
+        kv = torch.nn.functional.linear(cur, w).view(B, 2 * P, 2, H, Dh)
+        par = qkv[:, off:off + P].view(B, P, 3, H, Dh)
+        o = torch.empty(B, P, H, Dh, dtype=torch.bfloat16, device=DEV)
+        fn.build_parents_strided(par[:, :, 0], par[:, :, 1], par[:, :, 2], kv[:, :, 0], kv[:, :, 1], out=o)
+        cur = o.view(B, P, dim)
+        ref.append(cur)
+        off, P = off + P, P // 2
+    assert (got.float() - torch.cat(ref, dim=1).float()).abs().max() < 2e-2
+    top_knob(1)
+    with pytest.raises(sa.HsaError):
+        fn.cross_update_top(src, qkv, wp, torch.empty(B, C - 1, dim, dtype=torch.bfloat16, device=DEV), H)
+    lib = _lib.lib()
+    assert lib.hsa_cross_update_level_rows(B, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
+    top_knob(0)
+    assert lib.hsa_cross_update_level_rows(1, H, Dh, _lib.HSA_BF16) == 4096
+    assert lib.hsa_cross_update_level_rows(8, H, Dh, _lib.HSA_BF16) == 512
+    assert lib.hsa_cross_update_level_rows(4096, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
+    assert lib.hsa_cross_update_level_rows(1, 3, 24, _lib.HSA_BF16) == 0
+
+
+def test_cross_update_top_shapes_not_handled(top_knob):
+    top_knob(1)   # the single launch: more rows than it holds are refused
     assert fn.fused_top_rows(8, 64, torch.float32) == 0
     assert fn.fused_top_rows(3, 24, torch.bfloat16) == 0
     assert fn.fused_top_rows(8, 64, torch.bfloat16) == 64 and fn.fused_top_rows(8, 128, torch.bfloat16) == 32
