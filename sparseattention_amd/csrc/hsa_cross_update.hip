@@ -446,6 +446,7 @@ int hsa_cross_update_top_fwd(const void *src, const void *qkv, const void *w_kv,
     HSA_REQUIRE(src && qkv && w_kv && out, "null pointer");
     HSA_REQUIRE(B >= 1 && H >= 1 && Dh >= 1, "bad shape B=%d H=%d Dh=%d", B, H, Dh);
     HSA_REQUIRE(C >= 2 && hsa::ilog2_exact(C) >= 0, "row count must be a power of two >= 2 (got %d)", C);
+    HSA_REQUIRE(C <= (1 << 20) && H <= 65535, "C=%d or H=%d beyond what one grid covers", C, H);
     if (!hsa::top_shape_ok(H, Dh, dtype))
         return hsa::fail(HSA_ERR_UNSUPPORTED, "shape H=%d Dh=%d dtype=%d not handled by the fused levels", H, Dh, dtype);
     const int64_t Dm = (int64_t)H * Dh;
