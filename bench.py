@@ -150,11 +150,18 @@ def cpu_plumbing_case(oracle, cores):
 
 
 # ------------------------------------------------------------------------------------ cfg4
-def lm_forward_bench(args):
+LIB_LAUNCHERS = ("hsa_attn_fwd", "hsa_build_parents_fwd", "hsa_build_parents_strided_fwd", "hsa_cross_update_top_fwd",
+                 "hsa_build_tree_fwd", "hsa_span_input_y", "hsa_topology_device", "hsa_cross_update_pack_weights")
+
+
+def lm_forward_measure(steps, warmup):
     """cfg4: forward of the 6-layer decoder LM (d_model 512, 8 heads, FFN 2048 GELU, vocab 50257,
-    bf16, B=8, N=4096, window 16, random weights, token ids uniform over the vocabulary)."""
+    bf16, B=8, N=4096, window 16, random weights, token ids uniform over the vocabulary).  Returns
+    the forward time, the share of the two module calls (event pairs around them) and the GPU time
+    between event pairs put around every entry point of this library (its kernels alone)."""
     import torch
     import sparseattention_amd as sa
+    from sparseattention_amd import _lib
     from sparseattention_amd.modules import attention as attn_mod
 
     dev = torch.device("cuda:0")
@@ -163,38 +170,52 @@ def lm_forward_bench(args):
     model = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation="gelu", max_len=N)
     model = model.to(dev).to(torch.bfloat16).eval()
     tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(0)).to(dev)
-    K = min(args.steps, 20)
-    W = max(10, min(args.warmup, 20))  # the first forwards also grow the allocator's pools
+    K = min(steps, 20)
+    W = max(10, min(warmup, 20))  # the first forwards also grow the allocator's pools
     with torch.no_grad():
         for _ in range(W):
             model(tok)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(K):
-            model(tok)
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / K
+        reps = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(K):
+                model(tok)
+            torch.cuda.synchronize()
+            reps.append((time.perf_counter() - t0) * 1e3 / K)
+        ms = sorted(reps)[len(reps) // 2]
         # time share of the tree side (cross_update_Y: projections + one kernel per level) and of
         # the span attention op: the same forward with an event pair around each call
         spans = {"cross_update_Y": [], "hierarchical_attention": []}
         cls = attn_mod.HierarchicalAttention
         orig_c, orig_h = cls.cross_update_Y, attn_mod.hierarchical_attention
 
-        def timed(name, f):
+        def timed(store, f):
             def g(*a, **k):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
                 r = f(*a, **k)
                 e1.record()
-                spans[name].append((e0, e1))
+                store.append((e0, e1))
                 return r
             return g
 
-        cls.cross_update_Y = timed("cross_update_Y", orig_c)
-        attn_mod.hierarchical_attention = timed("hierarchical_attention", orig_h)
+        cls.cross_update_Y = timed(spans["cross_update_Y"], orig_c)
+        attn_mod.hierarchical_attention = timed(spans["hierarchical_attention"], orig_h)
         model(tok)
         torch.cuda.synchronize()
         cls.cross_update_Y, attn_mod.hierarchical_attention = orig_c, orig_h
+
+        # this library's launches alone: an event pair around every entry point that launches
+        handle = _lib.lib()
+        own, saved = [], {}
+        for name in LIB_LAUNCHERS:
+            saved[name] = getattr(handle, name)
+            setattr(handle, name, timed(own, saved[name]))
+        model(tok)
+        torch.cuda.synchronize()
+        for name, f in saved.items():
+            setattr(handle, name, f)
 
         # the same forward captured once into a HIP graph and replayed (no host work per launch);
         # a replay must reproduce the eager logits bit for bit, else the figure is not reported
@@ -219,17 +240,31 @@ def lm_forward_bench(args):
             if not torch.equal(captured, eager):
                 graph_ms = None
     share = {k: sum(a.elapsed_time(b) for a, b in v) for k, v in spans.items()}
+    own_ms = sum(a.elapsed_time(b) for a, b in own)
+    res = {"workload": "cfg4: decoder LM forward, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16, random init, eval mode",
+           "forward_ms": ms, "forward_ms_min": min(reps), "forward_ms_max": max(reps),
+           "tokens_per_s": B * N / (ms * 1e-3), "steps": K, "warmup": W, "repetitions": len(reps),
+           "ms_in_cross_update_Y_event_pairs": share["cross_update_Y"],
+           "ms_in_hierarchical_attention_event_pairs": share["hierarchical_attention"],
+           "share_cross_update_Y": share["cross_update_Y"] / ms,
+           "share_hierarchical_attention": share["hierarchical_attention"] / ms,
+           "ms_in_this_librarys_launches_event_pairs": own_ms, "launches_of_this_library": len(own),
+           "hip_graph_replay_ms_per_forward": graph_ms,
+           "calls_cross_update_Y": len(spans["cross_update_Y"]),
+           "calls_hierarchical_attention": len(spans["hierarchical_attention"])}
+    del model, tok, eager, captured, graph
+    torch.cuda.empty_cache()
+    return res
+
+
+def lm_forward_bench(args):
+    r = lm_forward_measure(args.steps, args.warmup)
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
-        "value": B * N / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
-        "config": {"workload": "cfg4: decoder LM forward, random init, eval mode"},
-        "detail": {"ms_in_cross_update_Y_event_pairs": share["cross_update_Y"],
-                   "ms_in_hierarchical_attention_event_pairs": share["hierarchical_attention"],
-                   "hip_graph_replay_ms_per_forward": graph_ms,
-                   "calls_cross_update_Y": len(spans["cross_update_Y"]),
-                   "calls_hierarchical_attention": len(spans["hierarchical_attention"])}}))
+        "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": r["steps"], "warmup": r["warmup"],
+        "ms_per_step": r["forward_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": r["workload"]}, "detail": r}))
 
 
 # ------------------------------------------------------------------------------------ GPU side
@@ -326,14 +361,15 @@ def between_events(torch, stream, K, launch):
     return e0.elapsed_time(e1) / K
 
 
-def kernel_times(torch, lib, hip, prob, stream, st, K, with_tree):
+def kernel_times(torch, lib, hip, prob, stream, st, K, with_tree, reps=15):
     """Durations on one stream, inputs rotated as in the timed steps:
       b2b   K span-attention launches one after the other between one pair of events: the average
             launch duration (an upper bound of the kernel's own: the launch gaps are inside);
+            repeated (see `repeated`), the median region counts;
       attn  the K steps once more with every attention dispatch carrying its own pair of HIP
             events (sorted); such a dispatch reads about 1 us longer than the same kernel in the
             rocprofv3 trace and than b2b;
-      tree  K tree builds between one pair of events."""
+      tree  K tree builds between one pair of events, repeated likewise."""
     n = len(prob.sets)
     targs = [prob.tree_args(s, st) for s in prob.sets]
     aargs = [prob.attn_args(s, st) for s in prob.sets]
@@ -349,11 +385,14 @@ def kernel_times(torch, lib, hip, prob, stream, st, K, with_tree):
     for a, b in kev:
         hip.free(a)
         hip.free(b)
-    b2b_ms = between_events(torch, stream, K, lambda i: lib.hsa_attn_fwd(*aargs[i % n]))
-    tree_ms = None
+    b2b = repeated(lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_fwd(*aargs[i % n])), K,
+                   min_reps=reps, min_total_ms=6.0)
+    tree = None
     if with_tree:
-        tree_ms = between_events(torch, stream, K, lambda i: lib.hsa_build_tree_fwd(*targs[i % n]))
-    return {"attn": attn, "b2b": b2b_ms, "tree": tree_ms}
+        tree = repeated(lambda: between_events(torch, stream, K, lambda i: lib.hsa_build_tree_fwd(*targs[i % n])), K,
+                        min_reps=reps, min_total_ms=6.0)
+    return {"attn": attn, "b2b": median(b2b), "tree": median(tree) if tree else None,
+            "b2b_samples": b2b, "tree_samples": tree}
 
 
 def wall_ms_per_step(torch, lib, prob, st_list, K, with_tree):
@@ -372,6 +411,21 @@ def wall_ms_per_step(torch, lib, prob, st_list, K, with_tree):
     t1 = time.perf_counter()
     assert rc == 0, lib.hsa_last_error()
     return (t1 - t0) * 1e3 / K
+
+
+def repeated(measure, K, min_reps=15, min_total_ms=12.0, max_reps=400):
+    """`measure()` times one region of K steps and returns ms per step.  Runs it at least
+    `min_reps` times and until the regions add up to `min_total_ms` of work, so that the figure
+    does not rest on a single sub-millisecond sample whatever K is; returns the sorted samples."""
+    xs = [measure()]
+    need = max(min_reps, int(min_total_ms / max(xs[0] * K, 1e-6)) + 1)
+    for _ in range(min(need, max_reps) - 1):
+        xs.append(measure())
+    return sorted(xs)
+
+
+def median(xs):
+    return xs[len(xs) // 2]
 
 
 def copy_reference(torch, stream, K, nbytes):
@@ -405,8 +459,8 @@ def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
     prob = Problem(torch, _lib, B, H, N, D, R, scale, causal, nsets, 1)
     for _ in range(2):
         wall_ms_per_step(torch, lib, prob, [st], min(K, 10), True)
-    step_ms = wall_ms_per_step(torch, lib, prob, [st], K, True)
-    kt = kernel_times(torch, lib, hip, prob, stream, st, K, True)
+    step_ms = median(repeated(lambda: wall_ms_per_step(torch, lib, prob, [st], K, True), K, min_reps=7, min_total_ms=6.0))
+    kt = kernel_times(torch, lib, hip, prob, stream, st, K, True, reps=7)
     attn, tree_ms, a_ms = kt["attn"], kt["tree"], kt["b2b"]
     e_ms = sum(attn) / len(attn)
     rec = {"workload": desc if causal else desc.replace("causal", "not causal"),
@@ -481,11 +535,16 @@ def main():
         wall_ms_per_step(torch, lib, prob, side_st, nsets, with_tree)
 
     # --- timed region: exactly K steps between two synchronisations -----------------------
-    ms_per_step = wall_ms_per_step(torch, lib, prob, side_st, K, with_tree)
+    #     The region is repeated (at least 15 times, and until 12 ms of work have been timed) and
+    #     the median region is reported: with --steps 20 a single region is 0.8 ms of work, and
+    #     one scheduler hiccup would move the figure by several per cent.
+    step_samples = repeated(lambda: wall_ms_per_step(torch, lib, prob, side_st, K, with_tree), K)
+    ms_per_step = median(step_samples)
 
     # --- the same K steps one after the other on a single stream (the latency of a step) ----
     wall_ms_per_step(torch, lib, prob, [st], min(args.warmup, 10), with_tree)
-    serial_ms_per_step = wall_ms_per_step(torch, lib, prob, [st], K, with_tree)
+    serial_samples = repeated(lambda: wall_ms_per_step(torch, lib, prob, [st], K, with_tree), K)
+    serial_ms_per_step = median(serial_samples)
 
     # --- duration of the dominant kernel, on one stream with the same rotation of inputs: K
     #     attention launches between one pair of events (the figure of the roofline object), the
@@ -508,13 +567,9 @@ def main():
               B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st) for s in prob.sets]
     for i in range(3):
         assert lib.hsa_attn_bwd(*bargs[i % nsets]) == 0, lib.hsa_last_error()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for i in range(K):
-        lib.hsa_attn_bwd(*bargs[i % nsets])
-    e1.record(stream)
-    torch.cuda.synchronize()
-    attn_bwd_ms = e0.elapsed_time(e1) / K
+    attn_bwd_ms = median(repeated(
+        lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd(*bargs[i % nsets])), K, min_reps=7,
+        min_total_ms=6.0))
     del gq, dq_, dk_, dv_, wsp
 
     # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
@@ -562,7 +617,12 @@ def main():
                                              "min_ms": attn_kernel_ms[0],
                                              "frac": attn_bytes / (attn_event_avg_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                              "timing": "the K steps once more, one stream, a HIP event pair attached to every attention dispatch (reads about 1 us more than the same dispatch in the rocprofv3 kernel trace)"}},
-        "detail": {"single_stream_ms_per_step": serial_ms_per_step,
+        "detail": {"timed_regions": {"regions_of_K_steps": len(step_samples), "reported": "median region",
+                                     "ms_per_step_min": step_samples[0], "ms_per_step_max": step_samples[-1],
+                                     "single_stream_ms_per_step_min": serial_samples[0],
+                                     "single_stream_ms_per_step_max": serial_samples[-1],
+                                     "attn_launch_ms_min": kt["b2b_samples"][0], "attn_launch_ms_max": kt["b2b_samples"][-1]},
+                   "single_stream_ms_per_step": serial_ms_per_step,
                    "single_stream_head_queries_per_s": head_queries / (serial_ms_per_step * 1e-3),
                    "step_algorithmic_bytes": step_algorithmic,
                    "step_GBps_two_streams": step_algorithmic / (ms_per_step * 1e-3) / 1e9,
@@ -597,7 +657,7 @@ def main():
         ns = sets_for(step_bytes(B, H, N, D, True), 0, 1)
         ao = Problem(torch, _lib, B, H, N, D, R, scale, causal, ns, 1, iid_nodes=True)
         wall_ms_per_step(torch, lib, ao, [st], 20, False)
-        ao_ms = wall_ms_per_step(torch, lib, ao, [st], K, False)
+        ao_ms = median(repeated(lambda: wall_ms_per_step(torch, lib, ao, [st], K, False), K, min_reps=7, min_total_ms=6.0))
         ao_k = kernel_times(torch, lib, hip, ao, stream, st, K, False)
         result["detail"]["attention_only_one_stream"] = {
             "ms_per_launch_wall_clock": ao_ms, "head_queries_per_s_wall_clock": head_queries / (ao_ms * 1e-3),
@@ -613,6 +673,8 @@ def main():
             "cfg3_noncausal": brief_config(torch, _lib, lib, hip, "cfg3", False, kb, 0.0),
             "cfg5": brief_config(torch, _lib, lib, hip, "cfg5", True, min(kb, 20), cs),
         }
+        # the decoder LM (its own metric: tokens/s of the forward; see --workload cfg4)
+        result["detail"]["configs"]["cfg4"] = lm_forward_measure(20, 10)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, H, N, D, R, causal, scale, args.cpu_seconds)
     if args.attention_only:

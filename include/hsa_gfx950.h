@@ -313,6 +313,10 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
  * refused with HSA_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's buffer: calls that
  * overlap on one GPU (two streams, two host threads) race; calls on one stream do not.
  * Nothing in the buffer has to be cleared between calls.
+ * The buffer's address on a GPU is looked up once per GPU: by hsa_attn_bwd_static_capacity() (the
+ * set-up call: make it once on every GPU before recording a graph there) or by the first
+ * hsa_attn_bwd_static on an ordinary stream.  A first use on a stream that is being captured is
+ * refused with HSA_ERR_UNSUPPORTED instead of doing the look-up inside the capture.
  */
 #define HSA_ATTN_BWD_STATIC_BYTES (32u << 20)
 size_t hsa_attn_bwd_static_capacity(void);

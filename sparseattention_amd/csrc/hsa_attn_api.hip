@@ -59,6 +59,8 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
     // offset) go to the gather kernel unless the tile kernel was asked for by name
     const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0;
     if (!aligned && algo != HSA_ATTN_TILE) tile_ok = false;
+    if (!aligned && algo == HSA_ATTN_TILE && tile_ok)
+        return hsa::fail(HSA_ERR_INVALID, "tile kernel needs 16-byte aligned tensors");
     if (algo == HSA_ATTN_TILE && !tile_ok)
         return hsa::fail(HSA_ERR_UNSUPPORTED,
                          "tile kernel not available for N=%d H=%d D=%d L=%d R=%d dtype=%d canonical=%d",

@@ -845,13 +845,21 @@ static constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mu;
 static void *g_scratch_ptr[kMaxDevices];  // per device, filled on the first call there
 
-static int scratch_for_current_device(void **out) {
+// `may_resolve` false: only an address that is already known is returned (a stream that is being
+// captured must not see the symbol lookup, which is no stream operation and may fail or end the
+// capture)
+static int scratch_for_current_device(void **out, bool may_resolve) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
     if (dev < 0 || dev >= kMaxDevices) return fail(HSA_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
     std::lock_guard<std::mutex> lock(g_scratch_mu);
     if (!g_scratch_ptr[dev]) {
+        if (!may_resolve)
+            return fail(HSA_ERR_UNSUPPORTED,
+                        "hsa_attn_bwd_static: first use on device %d while the stream is being captured; call "
+                        "hsa_attn_bwd_static_capacity() (or hsa_attn_bwd_static once) on this device before the capture",
+                        dev);
         void *p = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess || !p)
@@ -863,7 +871,13 @@ static int scratch_for_current_device(void **out) {
 }
 }  // namespace hsa
 
-size_t hsa_attn_bwd_static_capacity(void) { return (size_t)HSA_ATTN_BWD_STATIC_BYTES; }
+// Also the set-up call: resolves the buffer's address on the current device, so that a later
+// hsa_attn_bwd_static there does nothing but launch (what a captured stream needs).
+size_t hsa_attn_bwd_static_capacity(void) {
+    void *ws = nullptr;
+    (void)hsa::scratch_for_current_device(&ws, true);
+    return (size_t)HSA_ATTN_BWD_STATIC_BYTES;
+}
 
 int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
                         void *dv, int B, int N, int M, int H, int D, int L, int R, int causal, int dtype,
@@ -875,8 +889,13 @@ int hsa_attn_bwd_static(const void *q, const void *k, const void *v, const void 
         return hsa::fail(HSA_ERR_UNSUPPORTED,
                          "problem needs %zu bytes of scratch, the built-in buffer holds %zu: use hsa_attn_bwd "
                          "with a caller-provided workspace", need, (size_t)HSA_ATTN_BWD_STATIC_BYTES);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusNone;
+    }
     void *ws = nullptr;
-    const int rc = hsa::scratch_for_current_device(&ws);
+    const int rc = hsa::scratch_for_current_device(&ws, cap == hipStreamCaptureStatusNone);
     if (rc != HSA_OK) return rc;
     // the kernels write every workspace entry before they read it: nothing to clear between calls
     return hsa_attn_bwd(q, k, v, dout, dq, dk, dv, ws, (size_t)HSA_ATTN_BWD_STATIC_BYTES, B, N, M, H, D, L, R,

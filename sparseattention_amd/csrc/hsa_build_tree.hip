@@ -7,13 +7,16 @@
 //      2^TL leaves: every row it needs is requested up front, the TL levels stay in registers;
 //   B  a workgroup covers S consecutive subtrees of all H heads (so its wavefronts still read
 //      whole token rows); their roots are exchanged through LDS and the next log2 S levels are
-//      finished inside the workgroup (parent rows were requested together with phase A's);
+//      finished inside the workgroup (parent rows were requested together with phase A's and wait
+//      in LDS);
 //   C  what is left per batch element -- one node per workgroup -- is finished by "the last one to
 //      arrive": each workgroup publishes its node, increments an arrival counter shared by a group
 //      of 2^g neighbouring workgroups and exits unless it was the last of the group; the last one
 //      reads the group's 2^g nodes, computes g more levels and repeats one level of grouping
 //      further up, until the root.  Nobody spins: every workgroup exits after at most one pass
 //      over its own data plus the groups it happened to close.
+// The second copy of the result (out2) is written after the arrival: until then the launch is
+// almost purely reading, and the copy drains while the closing workgroups finish the top levels.
 // Arrival counters live in a device array that is part of the library image; they count with
 // wrap-around (the closing arrival resets the counter), so they are zero whenever no launch
 // is using them, and each stream has its own slice, so launches that may run concurrently
@@ -118,7 +121,9 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
     // (measured at B16 N512 .. B2 N4096, 8 heads of 64), while at 512 threads the launch gains
     // nothing and the span attention that follows loses the node rows the memory-side cache kept.
     constexpr bool STREAM = THREADS <= 256;
-    extern __shared__ __align__(16) unsigned char tree_lds[];
+    // LDS: two exchange buffers (2 * THREADS and THREADS pieces) and the staged parent rows
+    // (three tensors, 2 * THREADS pieces each): 144 bytes per thread
+    __shared__ __align__(16) unsigned char tree_lds[9 * THREADS * PB];
     unsigned char *bufX = tree_lds;                       // 2 * THREADS pieces
     unsigned char *bufY = tree_lds + 2 * THREADS * PB;    // THREADS pieces
     __shared__ int s_last;
@@ -145,24 +150,26 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
     auto node_row = [&](int level, int idx) { return (size_t)(level_offset(N, level) - N + idx) * rs; };
 
     // ---- phase A: TL levels in registers; every row is requested before the first use --------
-    // Requests go out in the order the results are used (level 1 parent by parent: its two
-    // children's K and V pieces and its own q/k/v; then the upper levels), and loads return in
-    // order: the arithmetic of the first parents runs while the later rows are still arriving.
+    // Requests go out tensor by tensor (a wavefront's eight leaf K rows are 8 KiB in a row, then
+    // the four level-1 q rows, ...): contiguous runs are served faster than the same rows
+    // requested in the order of use (measured on the bare request pattern at 8 x 2048 rows of
+    // 1 KiB: 12.6 against 13.4 us).  Loads return in order, so the first parents are computed
+    // while the upper levels' rows are still arriving.
     P rck[NC], rcv[NC], rq[NC - 1], rk[NC - 1], rv[NC - 1];
     {
         const S *kc = (const S *)a.kleaf + (size_t)b * a.kleaf_bs + (size_t)sub * NC * rs + hd;
         const S *vc = (const S *)a.vleaf + (size_t)b * a.vleaf_bs + (size_t)sub * NC * rs + hd;
         const size_t row1 = node_row(1, sub * (NC / 2));
 #pragma unroll
-        for (int i = 0; i < NC / 2; ++i) {
-            rq[i] = load_once<P>(Qp + row1 + (size_t)i * rs);
-            rck[2 * i] = load_once<P>(kc + (size_t)(2 * i) * rs);
-            rck[2 * i + 1] = load_once<P>(kc + (size_t)(2 * i + 1) * rs);
-            rk[i] = load_once<P>(Kp + row1 + (size_t)i * rs);
-            rcv[2 * i] = load_once<P>(vc + (size_t)(2 * i) * rs);
-            rcv[2 * i + 1] = load_once<P>(vc + (size_t)(2 * i + 1) * rs);
-            rv[i] = load_once<P>(Vp + row1 + (size_t)i * rs);
-        }
+        for (int i = 0; i < NC; ++i) rck[i] = load_once<P>(kc + (size_t)i * rs);
+#pragma unroll
+        for (int i = 0; i < NC / 2; ++i) rq[i] = load_once<P>(Qp + row1 + (size_t)i * rs);
+#pragma unroll
+        for (int i = 0; i < NC / 2; ++i) rk[i] = load_once<P>(Kp + row1 + (size_t)i * rs);
+#pragma unroll
+        for (int i = 0; i < NC; ++i) rcv[i] = load_once<P>(vc + (size_t)i * rs);
+#pragma unroll
+        for (int i = 0; i < NC / 2; ++i) rv[i] = load_once<P>(Vp + row1 + (size_t)i * rs);
     }
 #pragma unroll
     for (int j = 2; j <= TL; ++j) {
@@ -170,27 +177,35 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
         const int base = NC - 2 * np;
         const size_t row = node_row(j, sub * np);
 #pragma unroll
-        for (int i = 0; i < NC / 4; ++i) {
-            if (i < np) {
-                rq[base + i] = load_once<P>(Qp + row + (size_t)i * rs);
-                rk[base + i] = load_once<P>(Kp + row + (size_t)i * rs);
-                rv[base + i] = load_once<P>(Vp + row + (size_t)i * rs);
-            }
-        }
-    }
-    // phase B's parent rows: slot u_local serves parent p_local of every level where p_local is in
-    // range.  The loads are unconditional -- out-of-range slots re-read the level's last row and
-    // levels past the workgroup's last re-read that one -- because a load under a branch is
-    // waited for at the end of the branch, and with it every load requested before it.
-    P bq[TREE_NLMAX], bk[TREE_NLMAX], bv[TREE_NLMAX];
+        for (int i = 0; i < NC / 4; ++i)
+            if (i < np) rq[base + i] = load_once<P>(Qp + row + (size_t)i * rs);
 #pragma unroll
-    for (int j = 1; j <= TREE_NLMAX; ++j) {
-        const int je = j < lgS ? j : lgS;  // 0 when the workgroup holds one subtree: its root's row
-        const int np = 1 << (lgS - je);
-        const size_t row = node_row(TL + je, ((wg << lgS) >> je) + (p_local < np ? p_local : np - 1));
-        bq[j - 1] = load_once<P>(Qp + row);
-        bk[j - 1] = load_once<P>(Kp + row);
-        bv[j - 1] = load_once<P>(Vp + row);
+        for (int i = 0; i < NC / 4; ++i)
+            if (i < np) rk[base + i] = load_once<P>(Kp + row + (size_t)i * rs);
+#pragma unroll
+        for (int i = 0; i < NC / 4; ++i)
+            if (i < np) rv[base + i] = load_once<P>(Vp + row + (size_t)i * rs);
+    }
+    // phase B's parent rows, one piece per thread and tensor: thread t fetches what staging slot t
+    // holds (levels back to back, each level's (parent, head, lane) slots in order; the last
+    // H * G slots stay unused and re-read the top row).  The loads are unconditional, because a
+    // load under a branch is waited for at the end of the branch, and with it every load
+    // requested before it.
+    constexpr int LGT = ilog2_const(THREADS);
+    P sq, sk, sv;
+    {
+        const int m = THREADS - 1 - (int)threadIdx.x;
+        int jj = LGT - (31 - __clz(m | 1));     // slot t belongs to run level jj
+        jj = jj < lgS ? jj : lgS;
+        jj = jj > 0 ? jj : 0;                   // lgS == 0: no run; the subtree's own root row
+        const int first = jj > 0 ? THREADS - (THREADS >> (jj - 1)) : 0;
+        const int np = 1 << (lgS - jj);
+        int pp = ((int)threadIdx.x - first) >> (lgH + lgG);
+        pp = pp < np ? pp : np - 1;
+        const size_t row = node_row(TL + jj, ((wg << lgS) >> jj) + pp);
+        sq = load_once<P>(Qp + row);
+        sk = load_once<P>(Kp + row);
+        sv = load_once<P>(Vp + row);
     }
     // The parent rows of the levels above the workgroups' own (phase C) are read by whichever
     // workgroup closes a group, right after its arrival and on the critical path of the launch's
@@ -215,9 +230,11 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    // Every row is stored to `out` as it is produced and kept in registers for the second copy,
+    // which is written after the arrival (see `second_copy`).
+    P keep[NC - 1];
     {
         // level 1: keys and values are different rows
-        P lvl[NC / 2];
 #pragma unroll
         for (int i = 0; i < NC / 2; ++i) {
             float s0 = 0.f, s1 = 0.f, s2 = 0.f;
@@ -235,84 +252,141 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
             softmax3<T>(s0 * a.scale, s1 * a.scale, s2 * a.scale, w0, w1, w2);
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
-                lvl[i].e[e] = from_float<T>(w0 * to_float<T>(rv[i].e[e]) + w1 * to_float<T>(rcv[2 * i].e[e]) +
-                                            w2 * to_float<T>(rcv[2 * i + 1].e[e]));
-            const size_t row = node_row(1, sub * (NC / 2) + i);
-            store_node<STREAM>(Out + row, lvl[i]);
-            if (Out2) store_node<STREAM>(Out2 + row, lvl[i]);
+                keep[i].e[e] = from_float<T>(w0 * to_float<T>(rv[i].e[e]) + w1 * to_float<T>(rcv[2 * i].e[e]) +
+                                             w2 * to_float<T>(rcv[2 * i + 1].e[e]));
+            store_node<STREAM>(Out + node_row(1, sub * (NC / 2) + i), keep[i]);
         }
         // levels 2..TL
 #pragma unroll
         for (int j = 2; j <= TL; ++j) {
             const int np = NC >> j;
             const int base = NC - 2 * np;
+            const int cbase = NC - 4 * np;  // the level below
 #pragma unroll
             for (int i = 0; i < NC / 4; ++i) {
                 if (i < np) {
-                    const P r = combine<T, VEC>(rq[base + i], rk[base + i], rv[base + i], lvl[2 * i], lvl[2 * i + 1], G,
-                                                a.scale);
+                    const P r = combine<T, VEC>(rq[base + i], rk[base + i], rv[base + i], keep[cbase + 2 * i],
+                                                keep[cbase + 2 * i + 1], G, a.scale);
+                    keep[base + i] = r;
                     const size_t row = node_row(j, sub * np + i);
-                    if (j == TL && lgS == 0 && lg_wpb > 0) publish_piece(Out + row, r);
+                    if (j == TL && lgS == 0 && lg_wpb > 0) publish_piece(Out + row, r);  // the workgroup's node
                     else store_node<STREAM>(Out + row, r);
-                    if (Out2) store_node<STREAM>(Out2 + row, r);
-                    lvl[i] = r;
                 }
             }
         }
         // the subtree's root goes to LDS, slot = (subtree, head): piece threadIdx.x
-        *reinterpret_cast<P *>(bufX + (size_t)threadIdx.x * PB) = lvl[0];
+        *reinterpret_cast<P *>(bufX + (size_t)threadIdx.x * PB) = keep[NC - 2];
     }
 
-    // ---- phase B: lgS more levels inside the workgroup --------------------------------------
-    if (lgS > 0) lds_barrier();
+    // ---- phases B and C share one loop ----------------------------------------------------------
+    // A "run" finishes n_lds levels inside the workgroup: the children sit in LDS (bufX), the
+    // parents' q/k/v pieces wait in LDS as well (stg), one level per iteration of a loop that is
+    // not unrolled: phase B's levels and the levels of every closing stage of phase C are the
+    // same instructions.  A level costs a wavefront about 220 instructions; the levels of the
+    // launch's tail are bound by that (two wavefronts per SIMD at the first level of a stage:
+    // 1.1 us, one: 0.5 us), not by memory.
+    // Staging slot of (run level jj, thread t): w1x2 - (w1x2 >> (jj-1)) + t, where w1x2 is twice
+    // the number of lanes busy at the run's first level: levels back to back, so that slot s of
+    // the whole run is fetched by thread s mod THREADS (no row is fetched twice).
+    unsigned char *stgQ = tree_lds + 3 * THREADS * PB;   // 2 * THREADS pieces each
+    unsigned char *stgK = stgQ + 2 * THREADS * PB;
+    unsigned char *stgV = stgK + 2 * THREADS * PB;
+    *reinterpret_cast<P *>(stgQ + (size_t)threadIdx.x * PB) = sq;
+    *reinterpret_cast<P *>(stgK + (size_t)threadIdx.x * PB) = sk;
+    *reinterpret_cast<P *>(stgV + (size_t)threadIdx.x * PB) = sv;
+
+    // The second copy of phase A's rows.  Stored as they are produced, these writes compete with
+    // the reads that every workgroup still has under way; stored after the arrival they overlap
+    // the closing workgroups' top levels instead (headline shape: 28.7 -> 26 us per launch;
+    // deferring `out` as well loses again: the closing workgroups then work inside twice the
+    // write traffic).  A closing workgroup writes its own after its last stage.
+    auto second_copy = [&]() {
+        if (!Out2) return;
 #pragma unroll
-    for (int j = 1; j <= TREE_NLMAX; ++j) {
-        if (j <= lgS) {
-            const int np = 1 << (lgS - j);
-            unsigned char *src = (j & 1) ? bufX : bufY;
-            unsigned char *dst = (j & 1) ? bufY : bufX;
-            if (p_local < np) {
+        for (int j = 1; j <= TL; ++j) {
+            const int np = NC >> j;
+            const int base = NC - 2 * np;
+#pragma unroll
+            for (int i = 0; i < NC / 2; ++i)
+                if (i < np) store_node<STREAM>(Out2 + node_row(j, sub * np + i), keep[base + i]);
+        }
+    };
+
+    int n_lds = lgS;             // levels of the coming run
+    int lvl_base = TL;           // level of the run's children
+    int idx_base = wg << lgS;    // index (within the batch element) of the run's first child
+    int w1x2 = THREADS;          // twice the lanes busy at the run's first level
+    int level = TL + lgS;        // after the run this workgroup holds node `idx` of that level (all heads)
+    int idx = wg;
+    int lg_width = lg_wpb;       // nodes of that level per batch element (log2)
+    unsigned *cnt = a.counters + (size_t)b * a.counters_per_batch;
+    const int upb = THREADS >> lgG;  // (node, head) slots one pass of the workgroup covers
+    asm volatile("" : "+s"(n_lds));  // one copy of the loop for every run: nothing specialised for the first
+    if (n_lds > 0) lds_barrier();
+    for (;;) {
+        const bool more = lg_width > 0;  // another stage follows: the run's last level is published
+        unsigned char *src = bufX, *dst = bufY;
+#pragma unroll 1
+        for (int jj = 1; jj <= n_lds; ++jj) {
+            if ((int)threadIdx.x < (w1x2 >> jj)) {
+                const size_t slot = (size_t)(w1x2 - (w1x2 >> (jj - 1))) + threadIdx.x;
+                const P q = *reinterpret_cast<const P *>(stgQ + slot * PB);
+                const P k = *reinterpret_cast<const P *>(stgK + slot * PB);
+                const P v = *reinterpret_cast<const P *>(stgV + slot * PB);
                 const size_t c_off = ((size_t)(((2 * p_local) << lgH) + h) << lgG) + gl;
                 const P c0 = *reinterpret_cast<const P *>(src + c_off * PB);
                 const P c1 = *reinterpret_cast<const P *>(src + (c_off + ((size_t)1 << (lgH + lgG))) * PB);
-                const P r = combine<T, VEC>(bq[j - 1], bk[j - 1], bv[j - 1], c0, c1, G, a.scale);
-                const size_t row = node_row(TL + j, ((wg << lgS) >> j) + p_local);
-                if (j == lgS && lg_wpb > 0) publish_piece(Out + row, r);  // the workgroup's node
+                const P r = combine<T, VEC>(q, k, v, c0, c1, G, a.scale);
+                const size_t row = node_row(lvl_base + jj, (idx_base >> jj) + p_local);
+                if (jj == n_lds && more) publish_piece(Out + row, r);  // read by the stage that follows
                 else store_node<STREAM>(Out + row, r);
                 if (Out2) store_node<STREAM>(Out2 + row, r);
-                if (j < lgS) *reinterpret_cast<P *>(dst + (size_t)threadIdx.x * PB) = r;
+                if (jj < n_lds) *reinterpret_cast<P *>(dst + (size_t)threadIdx.x * PB) = r;
             }
-            if (j < lgS) lds_barrier();
+            if (jj < n_lds) lds_barrier();
+            unsigned char *t = src;
+            src = dst;
+            dst = t;
         }
-    }
+        if (!more) break;
 
-    asm volatile("" ::"v"(__builtin_bit_cast(VPackBits, touch).x));
-
-    // ---- phase C: the last workgroup of a group to arrive continues upwards ----------------
-    int level = TL + lgS;    // this workgroup holds node `idx` of that level (all heads)
-    int idx = wg;
-    int lg_width = lg_wpb;     // nodes of that level per batch element (log2)
-    unsigned *cnt = a.counters + (size_t)b * a.counters_per_batch;
-    const int upb = THREADS >> lgG;  // (node, head) slots one pass of the workgroup covers
-    while (lg_width > 0) {
+        // ---- arrival: the last workgroup of a group to arrive continues upwards ----------------
         const int g = lg_width < gcap ? lg_width : gcap;
         const int grp = idx >> g;
-        // this workgroup's node has been written with device-scope stores: once they have
-        // completed, count the arrival; the closing arrival wraps the counter back to zero
-        __builtin_amdgcn_s_waitcnt(0);
+        // This workgroup's node has been written with device-scope (sc1) stores, which the L2
+        // writes through to memory; such a store is acknowledged -- the wavefront's vmcnt drops --
+        // only when the write has reached the memory side, the point where every XCD's L2 misses
+        // meet.  So: wait for vmcnt = 0 in every wavefront, meet at the workgroup barrier, and only
+        // then count the arrival (a device-scope atomic, executed at the memory side as well).  The
+        // closing workgroup reads the nodes with device-scope (sc1) loads, which miss in its own
+        // L2, after it has seen the counter's closing value: it reads what the stores left.
+        // A release on the increment would be the portable spelling, but at device scope it makes
+        // the compiler write back the whole L2 (0.1 - 0.6 us per workgroup, serialised).  The
+        // wait is an asm statement with a memory clobber, so the compiler moves no store below it
+        // and no load above it; a second compiler barrier follows the "am I last" branch.
+        asm volatile("" ::"v"(__builtin_bit_cast(VPackBits, touch).x));  // keeps the touching load alive
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         if (threadIdx.x == 0) {
             const unsigned last = (1u << g) - 1u;
             s_last = atomicInc(cnt + grp, last) == last;
         }
         __syncthreads();
-        if (!s_last) return;
+        if (!s_last) {
+            second_copy();
+            return;
+        }
+        asm volatile("" ::: "memory");
 
-        // parents of every level of this stage, requested together with level 1's children
-        // (level 1 may take two passes over the slots, the levels above take one).  All loads
-        // are unconditional: slots and levels that do not exist re-read the nearest one.
+        // ---- the closing workgroup: the stage's first level from registers ----------------------
+        // Its children are the group's published nodes; it may take two passes over the slots.
+        // The parents of the levels above are requested together with them and staged in LDS for
+        // the run that follows.  All loads are unconditional: slots and levels that do not exist
+        // re-read the nearest one.
         const bool two = ((1 << (g - 1)) << lgH) > upb;
-        P cq[TREE_GCAP_MAX + 1], ckk[TREE_GCAP_MAX + 1], cvv[TREE_GCAP_MAX + 1], ch0[2], ch1[2];
+        P cq[2], ckk[2], cvv[2], ch0[2], ch1[2];
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u4 uq[2], uk[2], uv[2];
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
             const int p = (u_local + pass * upb) >> lgH;
@@ -326,15 +400,25 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
             ckk[pass] = *reinterpret_cast<const P *>(Kp + row);
             cvv[pass] = *reinterpret_cast<const P *>(Vp + row);
         }
+        // staging slots t and t + THREADS of the run that follows (levels 2..g of the stage)
+        const int lgw = g - 1 + lgH + lgG;   // log2 of w1x2
+        w1x2 = 1 << lgw;
 #pragma unroll
-        for (int j = 2; j <= TREE_GCAP_MAX; ++j) {
-            const int je = j < g ? j : g;
-            const int np = 1 << (g - je);
-            const int pc = p_local < np ? p_local : np - 1;
-            const size_t row = node_row(level + je, (grp << (g - je)) + pc);
-            cq[j] = *reinterpret_cast<const P *>(Qp + row);
-            ckk[j] = *reinterpret_cast<const P *>(Kp + row);
-            cvv[j] = *reinterpret_cast<const P *>(Vp + row);
+        for (int pass = 0; pass < 2; ++pass) {
+            const int sl = (int)threadIdx.x + pass * THREADS;
+            const int m = w1x2 - 1 - sl;
+            int jj = lgw - (31 - __clz((m > 0 ? m : 0) | 1));
+            jj = jj < g - 1 ? jj : g - 1;
+            jj = jj > 0 ? jj : 0;               // g == 1: no run; the stage's own parent row
+            const int first = jj > 0 ? w1x2 - (w1x2 >> (jj - 1)) : 0;
+            const int np = 1 << (g - 1 - jj);
+            int pp = (sl - first) >> (lgH + lgG);
+            pp = pp < np ? pp : np - 1;
+            pp = pp > 0 ? pp : 0;
+            const size_t row = node_row(level + 1 + jj, (grp << (g - 1 - jj)) + pp);
+            uq[pass] = *reinterpret_cast<const u4 *>(Qp + row);
+            uk[pass] = *reinterpret_cast<const u4 *>(Kp + row);
+            uv[pass] = *reinterpret_cast<const u4 *>(Vp + row);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -352,32 +436,23 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
                 }
             }
         }
-        if (g > 1) lds_barrier();
 #pragma unroll
-        for (int j = 2; j <= TREE_GCAP_MAX; ++j) {
-            if (j <= g) {
-                const int np = 1 << (g - j);
-                unsigned char *src = (j & 1) ? bufY : bufX;
-                unsigned char *dst = (j & 1) ? bufX : bufY;
-                if (p_local < np) {
-                    const size_t c_off = ((size_t)(((2 * p_local) << lgH) + h) << lgG) + gl;
-                    const P c0 = *reinterpret_cast<const P *>(src + c_off * PB);
-                    const P c1 = *reinterpret_cast<const P *>(src + (c_off + ((size_t)1 << (lgH + lgG))) * PB);
-                    const P r = combine<T, VEC>(cq[j], ckk[j], cvv[j], c0, c1, G, a.scale);
-                    const size_t row = node_row(level + j, (grp << (g - j)) + p_local);
-                    if (j == g && lg_width > g) publish_piece(Out + row, r);  // read by the next stage
-                    else store_node<STREAM>(Out + row, r);
-                    if (Out2) store_node<STREAM>(Out2 + row, r);
-                    if (j < g) *reinterpret_cast<P *>(dst + (size_t)threadIdx.x * PB) = r;
-                }
-                if (j < g) lds_barrier();
-            }
+        for (int pass = 0; pass < 2; ++pass) {
+            const size_t slot = (size_t)threadIdx.x + (size_t)pass * THREADS;
+            *reinterpret_cast<u4 *>(stgQ + slot * PB) = uq[pass];
+            *reinterpret_cast<u4 *>(stgK + slot * PB) = uk[pass];
+            *reinterpret_cast<u4 *>(stgV + slot * PB) = uv[pass];
         }
+        if (g > 1) lds_barrier();
+        n_lds = g - 1;
+        lvl_base = level + 1;
+        idx_base = grp << (g - 1);
         cnt += (size_t)1 << (lg_width - g);
         lg_width -= g;
         level += g;
         idx = grp;
     }
+    second_copy();  // the workgroups that closed the last stage (or a batch element's only workgroup)
 }
 
 // ---- arrival counters ------------------------------------------------------------------------
@@ -530,9 +605,8 @@ static int build_tree_fused_typed(const void *qp, const void *kp, const void *vp
         a.counters = cap != hipStreamCaptureStatusNone ? tree_counters_for_capture(per_batch * B) : tree_counter_slice(st);
         if (!a.counters) return HSA_ERR_UNSUPPORTED;
     }
-    const size_t lds = (size_t)3 * threads * 16;
 #define HSA_TREE_LAUNCH(THR, GG, HH) \
-    build_tree_fused_kernel<T, VEC, TL, THR, GG, HH><<<(unsigned)blocks, THR, lds, st>>>(a)
+    build_tree_fused_kernel<T, VEC, TL, THR, GG, HH><<<(unsigned)blocks, THR, 0, st>>>(a)
     // the common head layouts get their own instantiation at the two larger workgroup sizes
     const int key = lgG * 16 + lgH;
     if (threads == 512 && key == 3 * 16 + 3) HSA_TREE_LAUNCH(512, 3, 3);        // 8 heads, 8 lanes per row

@@ -348,7 +348,9 @@ static std::atomic<int> &top_single_launch() {
 
 // one launch per level reads the previous level's result rows 16 bytes at a time
 static bool top_levels_eligible(const TopParams &p) {
-    return !top_single_launch().load() && ((uintptr_t)p.out & 15) == 0 && p.out_rs % 8 == 0 && p.out_bs % 8 == 0;
+    // the per-level kernel moves 16-byte pieces of the children's rows and of the result rows
+    return !top_single_launch().load() && ((uintptr_t)p.out & 15) == 0 && p.out_rs % 8 == 0 && p.out_bs % 8 == 0 &&
+           ((uintptr_t)p.src & 15) == 0 && p.src_bs % 8 == 0 && p.Dm % 8 == 0;
 }
 
 template <typename T, int CT2, int PD>

@@ -37,14 +37,23 @@ class _SpanLevels(torch.autograd.Function):
     @staticmethod
     def forward(ctx, module, drop_p, x, y_in, wq, wk, wv):
         y_new, kept = module._span_levels(x, y_in, keep=True, drop_p=drop_p)
-        ctx.module, ctx.kept = module, kept
+        # everything the backward reads goes through save_for_backward: an in-place write to one
+        # of these tensors between forward and backward is then reported by autograd instead of
+        # giving wrong gradients, and saved-tensor hooks (checkpointing, offloading) see them
+        nl = len(kept["kvs"])
+        ctx.save_for_backward(kept["x"], kept["y_in"], kept["qkv"], kept["blocks"], kept["w_qkv"], kept["w_kv"],
+                              *kept["kvs"], *kept["masks"])
+        ctx.module, ctx.levels, ctx.scales = module, nl, kept["scales"]
         ctx.in_dtypes = (x.dtype, y_in.dtype, wq.dtype)
         return y_new
 
     @staticmethod
     def backward(ctx, dy):
-        dx, dy_in, dw = ctx.module._span_levels_backward(dy, ctx.kept)
-        ctx.kept = None
+        saved = ctx.saved_tensors  # raises autograd's own error if they were freed or modified
+        nl = ctx.levels
+        kept = dict(zip(("x", "y_in", "qkv", "blocks", "w_qkv", "w_kv"), saved[:6]))
+        kept["kvs"], kept["masks"], kept["scales"] = list(saved[6:6 + nl]), list(saved[6 + nl:]), ctx.scales
+        dx, dy_in, dw = ctx.module._span_levels_backward(dy, kept)
         xd, yd, wd = ctx.in_dtypes
         D = dx.shape[-1]
         dw = dw.to(wd)
@@ -178,7 +187,7 @@ class HierarchicalAttention(nn.Module):
         # child rows the fused upper levels take (0: shape not handled)
         # (y_new's rows are 16-byte aligned: the fused upper levels may run as a launch per level)
         top_rows = 0 if keep or not self.fuse_top_levels else _lib.lib().hsa_cross_update_level_rows(B, H, Dh, code)
-        kvs, masks = [], []
+        kvs, masks, scales = [], [], []
         src, off = x, 0
         with _lib.on_device(x):
             for lvl, P in enumerate(self.sizes):
@@ -194,13 +203,18 @@ class HierarchicalAttention(nn.Module):
                 kv = F.linear(src, w_kv)  # [B, 2P, 2D]
                 assert kv.dtype == cdt and kv.is_contiguous(), "projection result has an unexpected layout"
                 if drop_p > 0:
-                    # dropout on the value half, as a saved multiplicative mask
+                    # dropout on the value half: a saved boolean keep-mask (drawn in fp32) and one
+                    # scale applied as a scalar, i.e. in fp32 with a single rounding of the product
+                    # (a mask holding 1/keep_p in bf16 would scale by 1.109 instead of 1.111)
                     keep_p = 1.0 - drop_p
-                    m = torch.bernoulli(torch.full((B, 2 * P, D), keep_p, dtype=cdt, device=x.device)).div_(keep_p)
-                    if lvl == 0:
-                        m.mul_(torch.bernoulli(torch.full_like(m, keep_p)).div_(keep_p))
-                    kv[:, :, D:].mul_(m)
+                    m = torch.rand((B, 2 * P, D), dtype=torch.float32, device=x.device) < keep_p
+                    scale = 1.0 / keep_p
+                    if lvl == 0:  # the leaves' values pass through dropout twice
+                        m &= torch.rand((B, 2 * P, D), dtype=torch.float32, device=x.device) < keep_p
+                        scale = scale * scale
+                    kv[:, :, D:].mul_(m).mul_(scale)
                     masks.append(m)
+                    scales.append(scale)
                 par, kv_p, lvl_p = qkv_p + off * 3 * D * es, kv.data_ptr(), blk_p + B * off * D * es
                 rc = fwd(par, par + D * es, par + 2 * D * es, kv_p, kv_p + D * es, lvl_p,
                          out_p + off * D * es, B, P, H, Dh,
@@ -214,7 +228,7 @@ class HierarchicalAttention(nn.Module):
         if not keep:
             return y_new
         return y_new, {"x": x, "y_in": y_in, "qkv": qkv, "blocks": blocks, "kvs": kvs, "masks": masks,
-                       "w_qkv": w_qkv, "w_kv": w_kv}
+                       "scales": scales, "w_qkv": w_qkv, "w_kv": w_kv}
 
     def _span_levels_backward(self, dy: torch.Tensor, kept: dict):
         """Gradients of `_span_levels` with respect to x, y_in and the stacked q|k|v weights:
@@ -248,7 +262,7 @@ class HierarchicalAttention(nn.Module):
                          A(P * D, T3, T3, T3, 4 * P * D, 4 * P * D, T3, T3, T3, 4 * P * D, 4 * P * D), rs, code, stream)
                 _lib.check(rc, "hsa_build_parents_strided_bwd")
                 if masks:
-                    dkv[:, :, D:].mul_(masks[lvl])
+                    dkv[:, :, D:].mul_(masks[lvl]).mul_(kept["scales"][lvl])
                 src = x if lvl == 0 else blocks[B * self.offsets[lvl - 1] * D:B * off * D].view(B, 2 * P, D)
                 dw_kv += torch.matmul(dkv.reshape(-1, 2 * D).t(), src.reshape(-1, D)).float()
                 d_src = torch.matmul(dkv, w_kv)  # [B, 2P, D]

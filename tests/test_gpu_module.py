@@ -10,6 +10,7 @@ import torch
 import torch.nn as nn
 
 import oracle
+from conftest import error_figures, report
 import sparseattention_amd as sa
 
 pytestmark = pytest.mark.gpu
@@ -17,6 +18,7 @@ DEV = "cuda:0"
 
 
 def _within(got, want, atol, rtol, what):
+    report(what, **error_figures(got, want))
     got, want = got.detach().double().cpu(), want.double()
     err = (got - want).abs()
     bad = err > atol + rtol * want.abs()
@@ -36,10 +38,9 @@ def test_lm_at_benchmark_width_vs_oracle(dtype):
     """d_model 512, 8 heads of 64, FFN 2048 GELU, window 16 — the layer shape of the decoder-LM
     benchmark configuration — on 512 tokens, so that the strided levels, the fused upper levels
     (64 child rows) and the MFMA span attention all run, two layers deep, in 16-bit.  Compared with
-    the fp64 oracle on the rounded weights.  Tolerance: the 16-bit bar (2e-2 abs + 1e-2 rel) once
-    per residual stage that rounds (embedding, two per layer, read-out) — and, as a scale-free
-    cross-check, the error must stay within 3x the error the oracle's own algorithm makes when it
-    is evaluated in the same 16-bit type with torch on the CPU."""
+    the fp64 oracle on the rounded weights.  Tolerance: 2.5 x the measured max-abs error — and, as a
+    scale-free cross-check, the error must stay within 3x the error the oracle's own algorithm
+    makes when it is evaluated in the same 16-bit type with torch on the CPU."""
     V, d, H, ff, layers, N, B, R = 1000, 512, 8, 2048, 2, 512, 2, 16
     torch.manual_seed(0)
     m = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation="gelu", max_len=N).eval()
@@ -50,8 +51,9 @@ def test_lm_at_benchmark_width_vs_oracle(dtype):
         got = md(tok.to(DEV))
     assert got.dtype == dtype and got.shape == (B, N, V)
     want = oracle.lm_forward_ref(sd, tok, H, layers, R, "gelu", dtype=torch.float64)
-    stages = 2 + 2 * layers
-    _within(got, want, 2e-2 * stages, 1e-2 * stages, "LM logits %s" % dtype)
+    # measured max-abs error of the logits (size up to 6.4): 2.0e-2 in bf16, 2.5e-3 in fp16;
+    # bar = 2.5 x that, no relative term
+    _within(got, want, 5e-2 if dtype == torch.bfloat16 else 6.5e-3, 0.0, "LM logits %s" % dtype)
     low = oracle.lm_forward_ref({k: v.to(dtype) if v.is_floating_point() else v for k, v in sd.items()},
                                 tok, H, layers, R, "gelu", dtype=dtype)
     e_kernel = float((got.double().cpu() - want).abs().max())
@@ -113,9 +115,10 @@ def test_module_at_benchmark_width_vs_oracle(causal):
         y_new = m.cross_update_Y(x.to(DEV), y.to(DEV))
         mask = torch.ones(1, dtype=torch.bool, device=DEV) if causal else None
         out = m(x.to(DEV), x.to(DEV), x.to(DEV), y=y.to(DEV), mask=mask)
-    # three rounding stages each (projection, op, output projection)
-    _within(y_new, oracle.cross_update_y_ref(x.double(), y.double(), w, H), 3e-2, 1e-2, "cross_update_Y")
-    _within(out, oracle.update_x_from_y_ref(x.double(), y.double(), w, H, R, causal), 3e-2, 1e-2, "forward")
+    # three rounding stages each (projection, op, output projection); measured max-abs error
+    # 3.0e-3 / 2.4e-3 on outputs of size 0.7; bar = 2.5 x that, no relative term
+    _within(y_new, oracle.cross_update_y_ref(x.double(), y.double(), w, H), 8e-3, 0.0, "cross_update_Y")
+    _within(out, oracle.update_x_from_y_ref(x.double(), y.double(), w, H, R, causal), 6e-3, 0.0, "forward")
 
 
 # ---------------------------------------------------------------- the reference's own two check configurations
@@ -224,8 +227,8 @@ def test_module_under_autocast(amp, N, direct):
         y_new = m.cross_update_Y(x.to(DEV), y.to(DEV))
         out = m(x.to(DEV), x.to(DEV), x.to(DEV), y=y.to(DEV), mask=mask)
     assert y_new.dtype == amp and out.dtype == amp
-    _within(y_new, oracle.cross_update_y_ref(x.double(), y.double(), w, H), 3e-2, 1e-2, "cross_update_Y")
-    _within(out, oracle.update_x_from_y_ref(x.double(), y.double(), w, H, R, True), 3e-2, 1e-2, "forward")
+    _within(y_new, oracle.cross_update_y_ref(x.double(), y.double(), w, H), 8e-3, 0.0, "cross_update_Y")
+    _within(out, oracle.update_x_from_y_ref(x.double(), y.double(), w, H, R, True), 8e-3, 0.0, "forward")
     # and with autograd on (the training step runs under autocast as well)
     with torch.autocast("cuda", dtype=amp):
         y_tr = m.cross_update_Y(x.to(DEV), y.to(DEV))
@@ -398,8 +401,10 @@ def test_fused_span_node_update_with_dropout():
         y_plain, _ = m._span_levels(x.detach(), y.detach(), keep=True, drop_p=0.0)
     y_new, kept = m._span_levels(x.detach(), y.detach(), keep=True, drop_p=p)
     assert (y_new - y_plain).abs().max() > 1e-3
-    masks = [mk.double().cpu() for mk in kept["masks"]]
-    assert len(masks) == len(m.sizes) and all(((mk == 0) | (mk > 1)).all() for mk in masks)
+    assert all(mk.dtype == torch.bool for mk in kept["masks"])
+    assert kept["scales"][0] == (1 / (1 - p)) ** 2 and all(sc == 1 / (1 - p) for sc in kept["scales"][1:])
+    masks = [mk.double().cpu() * sc for mk, sc in zip(kept["masks"], kept["scales"])]
+    assert len(masks) == len(m.sizes)
     frac0 = float((masks[0] == 0).double().mean())
     assert abs(frac0 - (1 - (1 - p) ** 2)) < 0.05          # two rounds of dropout on the leaves' values
     # the same computation in fp64 with the masks put in by hand
@@ -426,6 +431,45 @@ def test_fused_span_node_update_with_dropout():
     out = m.cross_update_Y(x, y)
     out.square().mean().backward()
     assert x.grad is not None and y.grad is not None and m.Wv_y.weight.grad is not None
+
+
+def test_fused_span_node_update_saved_tensors():
+    """The fused training function keeps its activations through save_for_backward: a second
+    backward (retain_graph) reproduces the first, and an in-place write to an input between
+    forward and backward is reported by autograd, as it is for the reference's Linear layers."""
+    B, N, dim, H = 2, 16, 64, 2
+    torch.manual_seed(5)
+    m = sa.HierarchicalAttention(dim, H, dropout=0.0, window_size=4).to(DEV).train()
+    x = torch.randn(B, N, dim, device=DEV).requires_grad_(True)
+    y = torch.randn(B, N - 1, dim, device=DEV).requires_grad_(True)
+    loss = m.cross_update_Y(x, y).square().mean()
+    loss.backward(retain_graph=True)
+    g1 = x.grad.clone()
+    x.grad = None
+    loss.backward()
+    assert torch.equal(g1, x.grad)
+    xl = torch.randn(B, N, dim, device=DEV)          # a leaf the function saves as it is
+    loss = m.cross_update_Y(xl, y).square().mean()
+    xl.add_(1.0)
+    with pytest.raises(RuntimeError, match="modified by an inplace operation"):
+        loss.backward()
+
+
+def test_fused_span_node_update_dropout_scale_bf16():
+    """The dropout scale is applied in fp32 with one rounding: in bf16 the kept values equal the
+    undropped ones times 1/keep_p rounded once (a bf16 mask value would be off by 0.3 %)."""
+    B, N, dim, H, p = 1, 8, 64, 2, 0.1
+    torch.manual_seed(9)
+    m = sa.HierarchicalAttention(dim, H, dropout=p, window_size=2).to(DEV).to(torch.bfloat16).train()
+    x = torch.randn(B, N, dim, device=DEV, dtype=torch.bfloat16)
+    y = torch.randn(B, N - 1, dim, device=DEV, dtype=torch.bfloat16)
+    m.sizes, m.offsets = m._build_level_info(N)
+    _, kept = m._span_levels(x, y, keep=True, drop_p=p)
+    w_kv = kept["w_kv"]
+    src = kept["blocks"][:B * (N // 2) * dim].view(B, N // 2, dim)       # level 1's rows feed level 2
+    plain = torch.nn.functional.linear(src, w_kv)[:, :, dim:]
+    want = (plain.float() * kept["masks"][1] * kept["scales"][1]).to(torch.bfloat16)
+    assert torch.equal(kept["kvs"][1][:, :, dim:], want)
 
 
 # ---------------------------------------------------------------- the reference's import name

@@ -9,6 +9,7 @@ import torch
 
 import oracle
 import sparseattention_amd as sa
+from conftest import error_figures, report
 from sparseattention_amd import _lib
 from sparseattention_amd.ops import functional as fn
 
@@ -304,7 +305,9 @@ def test_cross_update_top_levels(B, C, H, Dh, dtype, single, top_knob):
         want.append(cur)
         off, P = off + P, P // 2
     want = torch.cat(want, dim=1)
-    assert (got.double().cpu() - want).abs().max() < 3e-2
+    report("cross_update_top_levels %s" % ((B, C, H, Dh, str(dtype), single),), **error_figures(got, want))
+    # measured max-abs error: 8.4e-3 (bf16), 9.4e-4 (fp16) over these shapes; bar = 2.5 x that
+    assert (got.double().cpu() - want).abs().max() < (2.1e-2 if dtype == torch.bfloat16 else 2.4e-3)
     # level by level on the GPU (each level's projection rounded to the element type, as here)
     cur, off, P, ref = src.to(DEV), 0, C // 2, []
     while P >= 1:
@@ -545,7 +548,10 @@ def test_module_vs_oracle(dtype, causal):
         mask = torch.ones(B, N, dtype=torch.bool, device=DEV) if causal else None
         out = md(xd, xd, xd, y=yd, mask=mask)
         want = oracle.update_x_from_y_ref(xr, yr, wr, H, R, causal)
-    atol = 1e-4 if dtype == torch.float32 else 3e-2   # GEMM chains; the reference's own bar is 1e-2..5e-2
+    # GEMM chains (the reference's own bar is 1e-2..5e-2); measured max-abs error in bf16: 2.3e-3
+    # (fp32: 3e-7); bar = 2.5 x that
+    atol = 1e-4 if dtype == torch.float32 else 6e-3
+    report("module_vs_oracle %s causal=%s" % (dtype, causal), y=error_figures(y_new, want_y), out=error_figures(out, want))
     assert (y_new.double().cpu() - want_y).abs().max() < atol
     assert (out.double().cpu() - want).abs().max() < atol
     assert md(xd, xd, xd, y=yd, mask=mask, return_attention=True)[1] is None
@@ -572,11 +578,15 @@ def test_module_fused_projection_path_matches_level_by_level_path(dtype, N, dim,
     stepwise = m.cross_update_Y(x.requires_grad_(True), y)
     assert stepwise.requires_grad and not fused.requires_grad
     assert torch.equal(fused, again) and torch.equal(fused, third)
-    tol = 1e-5 if dtype == torch.float32 else 3e-2
+    # measured in bf16: 2.5e-3 against the oracle, 2.0e-3 (one rounding step) between the paths;
+    # bar = 2.5 x that
+    tol = 1e-5 if dtype == torch.float32 else 6e-3
     assert (fused.float() - stepwise.detach().float()).abs().max() < tol
     w = {k: v.detach().double().cpu() for k, v in m.state_dict().items()}
     want = oracle.cross_update_y_ref(x.detach().double().cpu(), y.double().cpu(), w, H)
-    assert (fused.double().cpu() - want).abs().max() < (1e-4 if dtype == torch.float32 else 3e-2)
+    report("module_fused_vs_stepwise %s N=%d dim=%d" % (dtype, N, dim), oracle=error_figures(fused, want),
+           paths=error_figures(fused, stepwise))
+    assert (fused.double().cpu() - want).abs().max() < (1e-4 if dtype == torch.float32 else 6e-3)
     m.fuse_top_levels = False
     with torch.no_grad():
         unfused_top = m.cross_update_Y(x.detach(), y)
@@ -589,6 +599,33 @@ def _bf_check(bf, q, k, v, N, R, causal, out, dtype):
     want = bf.attention(q.float().numpy(), k.float().numpy(), v.float().numpy(), o["forward_idx"],
                         o["forward_mask"] if causal else None, R)
     assert_close(out, torch.from_numpy(want), dtype, "full-size")
+    return error_figures(out, torch.from_numpy(want)), torch.from_numpy(want)
+
+
+def _north_star_bars(f, what, low=None):
+    """The two bf16 bars, each on its own.  Max-abs <= 2e-2 holds everywhere and is asserted as
+    it stands.  Max-rel <= 1e-2 (over the elements whose reference is at least 0.1 in size) is
+    asserted where it holds; on N(0,1) inputs it cannot: an output near 0.1 is a sum of terms of
+    size 1, each weight rounded to bf16 (relative 2^-9) as in the reference's own arithmetic, so
+    absolute errors of 1..2e-3 are relative errors of 1..2e-2 there.  In that case `low` holds
+    the figures of the reference's algorithm evaluated in bf16 by torch on the same inputs, and
+    the kernel must be at least as close to the fp64 result as that."""
+    assert f["max_abs"] <= 2e-2, "%s: max abs err %.3e" % (what, f["max_abs"])
+    if low is None:
+        assert f["max_rel"] <= 1e-2, "%s: max rel err %.3e" % (what, f["max_rel"])
+    else:
+        assert f["max_abs"] <= low["max_abs"] and f["max_rel"] <= max(1e-2, low["max_rel"]), \
+            "%s: kernel %s vs the reference's algorithm in bf16 %s" % (what, f, low)
+
+
+def _bf16_reference_figures(q, k, v, N, R, causal, want):
+    """Error figures of the reference's algorithm evaluated in bf16 by torch on the CPU (gather,
+    einsum, softmax, einsum: every stage rounds to bf16) against `want`, on the first two batch
+    elements."""
+    o = oracle.topology_tables(N, causal)
+    low = oracle.attention_ref(q[:2], k[:2], v[:2], o["forward_idx"], o["forward_mask"] if causal else None, R)
+    assert low.dtype == torch.bfloat16
+    return error_figures(low, want[:2])
 
 
 @pytest.mark.parametrize("causal", [True, False])
@@ -799,7 +836,9 @@ def test_cfg2_tile_full_size(causal, bf):
     t = sa.build_tree_topology(N, causal, device=DEV)
     out = sa.hierarchical_attention(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"], t["backward_gather"],
                                     t["forward_mask"] if causal else None, R)
-    _bf_check(bf, q, k, v, N, R, causal, out, torch.bfloat16)
+    f, _ = _bf_check(bf, q, k, v, N, R, causal, out, torch.bfloat16)
+    report("cfg2_tile_full_size causal=%s" % causal, **f)
+    _north_star_bars(f, "cfg2")
 
 
 @pytest.mark.parametrize("causal", [True, False])
@@ -820,7 +859,14 @@ def test_cfg3_headline_full_size(causal, bf):
     t = sa.build_tree_topology(N, causal, device=DEV)
     out = sa.hierarchical_attention(q.to(DEV), kfull, vfull, t["forward_idx"], t["backward_gather"],
                                     t["forward_mask"] if causal else None, R)
-    _bf_check(bf, q, kfull.cpu(), vfull.cpu(), N, R, causal, out, torch.bfloat16)
+    f, want = _bf_check(bf, q, kfull.cpu(), vfull.cpu(), N, R, causal, out, torch.bfloat16)
+    low = _bf16_reference_figures(q, kfull.cpu(), vfull.cpu(), N, R, causal, want)
+    f_tree = error_figures(kfull[:, N:], tree)
+    low_tree = error_figures(oracle.build_tree_ref(qp[:2], kp[:2], vp[:2], kl[:2], vl[:2]), tree[:2])
+    report("cfg3_headline_full_size causal=%s" % causal, tree=f_tree, reference_in_bf16=low,
+           reference_tree_in_bf16=low_tree, **f)
+    _north_star_bars(f, "cfg3", low)
+    _north_star_bars(f_tree, "cfg3 tree", low_tree)
     out_g = fn.attention_forward(q.to(DEV), kfull, vfull, t["forward_idx"],
                                  t["forward_mask"] if causal else None, R, algo="gather")
     assert (out.float() - out_g.float()).abs().max() < 2e-2
@@ -879,6 +925,18 @@ def test_long_sequence_properties(shape):
         outs.append(torch.einsum("hs,shd->hd", p, vf))
     want = torch.stack(outs).unsqueeze(0)
     assert_close(out[:, sel], want, torch.bfloat16, "cfg5 sampled rows")
+    f = error_figures(out[:, sel], want)
+    assert f["max_abs"] <= 2e-2
+    # the last 512 queries in full: the kernel against the fp64 oracle, beside the reference's
+    # algorithm evaluated in bf16 by torch against the same
+    lo, hi = N - 512, N
+    blk = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"], R, compute_dtype=torch.float64,
+                               query_range=(lo, hi))[:, lo:hi]
+    low = error_figures(oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"], R,
+                                             query_range=(lo, hi))[:, lo:hi], blk)
+    f_blk = error_figures(out[:, lo:hi], blk)
+    report("long_sequence_properties %s" % (shape,), sampled_rows=f, last_512_queries=f_blk, reference_in_bf16=low)
+    _north_star_bars(f_blk, "long sequence, last 512 queries", low)
     # the gather kernel agrees with the tile kernel at this size
     og = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R, algo="gather")
     assert (og.float() - out.float()).abs().max() < 2e-2

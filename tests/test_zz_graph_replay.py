@@ -125,3 +125,42 @@ def test_lm_forward_replays_from_a_hip_graph():
             want = model(tok)
             torch.cuda.synchronize()
             assert torch.equal(got, want), "replay %d differs" % rep
+
+
+def test_lm_full_benchmark_shape_properties():
+    """The decoder-LM benchmark configuration at its FULL shape (6 layers, d_model 512, 8 heads,
+    FFN 2048 GELU, vocabulary 50257, bf16, batch 8, 4096 tokens, window 16, random weights): too
+    large for the CPU oracle, so what the model's definition fixes is checked: finite logits;
+    causality (changing the token at position n leaves the logits of every earlier position bit
+    for bit as they were, and changes position n); a HIP-graph replay of the forward reproduces
+    the eager logits bit for bit."""
+    torch.manual_seed(0)
+    V, d, H, ff, layers, N, B, R = 50257, 512, 8, 2048, 6, 4096, 8, 16
+    model = sa.TransformerLM(V, d, H, ff, layers, dropout=0.0, window_size=R, activation="gelu", max_len=N)
+    model = model.to(DEV).to(torch.bfloat16).eval()
+    tok = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(0)).to(DEV)
+    with torch.no_grad():
+        base = model(tok)
+        assert base.shape == (B, N, V) and base.dtype == torch.bfloat16
+        assert bool(torch.isfinite(base).all())
+        n = 2500
+        tok2 = tok.clone()
+        tok2[:, n] = (tok2[:, n] + 1) % V
+        other = model(tok2)
+        assert torch.equal(other[:, :n], base[:, :n]), "a later token changed earlier logits"
+        assert not torch.equal(other[:, n], base[:, n])
+        del other
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model(tok)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = model(tok)
+        for rep in range(2):
+            out.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, base), "replay %d differs from the eager forward" % rep

@@ -76,3 +76,41 @@ def test_static_scratch_backward_fp32_and_limit():
     rc = lib.hsa_attn_bwd_static(*([_lib.ptr(dummy)] * 7), B, N, M, H, D, L, R, 1, 2, 0, _lib.stream_of(dummy))
     assert rc == -95
     assert b"scratch" in lib.hsa_last_error()
+
+
+def test_static_scratch_backward_records_into_a_graph():
+    """After the set-up call the static entry is nothing but kernel launches: it can be recorded
+    into a HIP graph; every replay (with eager work and synchronisations in between) reproduces
+    the eager gradients bit for bit."""
+    lib = _lib.lib()
+    assert lib.hsa_attn_bwd_static_capacity() > 0          # resolves the buffer's address on this GPU
+    B, N, H, D, R, dtype = 2, 512, 4, 64, 16, torch.bfloat16
+    q, k, v, go = (t.to(DEV) for t in _inputs(B, N, H, D, dtype, seed=7))
+    L, M = N.bit_length() - 1, 2 * N - 1
+    code = _lib.dtype_code(q)
+    outs = [torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)]
+
+    def call():
+        rc = lib.hsa_attn_bwd_static(_lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(go), *map(_lib.ptr, outs),
+                                     B, N, M, H, D, L, R, 1, code, 0, _lib.stream_of(q))
+        _lib.check(rc, "hsa_attn_bwd_static")
+
+    call()
+    torch.cuda.synchronize()
+    want = [t.clone() for t in outs]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        for t in outs:
+            t.fill_(float("nan"))      # eager work between the replays (a fill kernel, no memset node)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, w, g in zip(("dQ", "dK", "dV"), want, outs):
+            assert torch.equal(w, g), "%s differs on replay %d" % (name, rep)
