@@ -303,6 +303,31 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
                  int L, int R, int causal, int dtype, int algo, void *stream);
 
 /*
+ * Span attention backward in one pass, for callers that kept two pieces of forward state, as the
+ * reference's autograd Function keeps its Weights tensor for the same purpose
+ * (hierarchical_attention/ops/functional.py:163-167, 171-264; kernels ops/triton/sparse_attn.py:185-623):
+ *   out  [B, N, H, D]  the forward's output
+ *   lse  [B, N, H] fp32 the log-sum-exp of every (query, head)'s biased logits in the log2 domain,
+ *                      written by hsa_attn_fwd_lse
+ * With them a strip of queries also finishes the gradients of its own leaf keys (what the
+ * neighbouring strips' queries add is rebuilt from their Q, dO rows, lse and delta = <dO, out>),
+ * so Q, dO, K, V are read once instead of twice.  Same results as hsa_attn_bwd to the rounding of
+ * the element type; deterministic.  Canonical tables only; fp16 / bf16, 32 or 64 channels per
+ * head, window radius up to 16, N >= 64, 16-byte aligned tensors: anything else returns
+ * HSA_ERR_UNSUPPORTED (hsa_attn_bwd_saved_workspace_bytes returns 0) and the caller uses
+ * hsa_attn_bwd.  workspace: hsa_attn_bwd_saved_workspace_bytes(...) bytes, written before read.
+ *
+ * hsa_attn_fwd_lse: hsa_attn_fwd on the canonical tables that also writes lse (16-bit tile kernel
+ * only; HSA_ERR_UNSUPPORTED otherwise, nothing launched).
+ */
+int hsa_attn_fwd_lse(const void *q, const void *k, const void *v, void *out, float *lse, int B, int N, int M,
+                     int H, int D, int L, int R, int causal, int dtype, void *stream);
+size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype);
+int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *out, const float *lse,
+                       const void *dout, void *dq, void *dk, void *dv, void *workspace, size_t workspace_bytes,
+                       int B, int N, int M, int H, int D, int L, int R, int causal, int dtype, void *stream);
+
+/*
  * hsa_attn_bwd for callers that cannot allocate device memory or hand over a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference: its backward allocates its workspaces through torch

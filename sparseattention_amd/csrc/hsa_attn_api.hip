@@ -9,7 +9,7 @@ int attn_gather_dispatch(const void *q, const void *k, const void *v, const int3
 
 bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, bool canonical,
                         bool want_weights, bool causal);
-int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
+int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, float *lse, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st);
 int attn_tile_tune(int sb, int wpb, int swizzle, int alternate);
 bool attn_tile_f32_eligible(int N, int M, int D, int L, int R, bool canonical, bool want_weights);
@@ -74,7 +74,7 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
             if (ev.start && ev.stop) (void)hipEventRecord(ev.stop, st);
             return rc;
         }
-        return hsa::attn_tile_dispatch(q, k, v, out, weights, B, N, M, H, D, L, R, causal ? 1 : 0, dtype, st);
+        return hsa::attn_tile_dispatch(q, k, v, out, weights, nullptr, B, N, M, H, D, L, R, causal ? 1 : 0, dtype, st);
     }
     // the gather kernels take no dispatch events: record around the call instead
     const hsa::LaunchEvents ev = hsa::take_launch_events();
@@ -83,6 +83,20 @@ int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx
                                              causal ? 1 : 0, dtype, st);
     if (ev.start && ev.stop) (void)hipEventRecord(ev.stop, st);
     return rc;
+}
+
+int hsa_attn_fwd_lse(const void *q, const void *k, const void *v, void *out, float *lse, int B, int N, int M,
+                     int H, int D, int L, int R, int causal, int dtype, void *stream) {
+    HSA_REQUIRE(q && k && v && out && lse, "null pointer");
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
+    HSA_REQUIRE(L >= 0 && R >= 0, "bad L=%d R=%d", L, R);
+    if ((dtype != HSA_F16 && dtype != HSA_BF16) ||
+        !hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, true, false, causal != 0) ||
+        ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output comes from the 16-bit tile kernel only "
+                         "(N=%d H=%d D=%d L=%d R=%d dtype=%d)", N, H, D, L, R, dtype);
+    return hsa::attn_tile_dispatch(q, k, v, out, nullptr, lse, B, N, M, H, D, L, R, causal ? 1 : 0, dtype,
+                                   (hipStream_t)stream);
 }
 
 int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_t *idx,

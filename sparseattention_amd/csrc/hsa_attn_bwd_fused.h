@@ -1,0 +1,568 @@
+// Span attention backward in ONE pass over the strips (16-bit element types, canonical tables,
+// window radius up to 16), for callers that kept the forward's output and log-sum-exp.
+//
+// The two-pass split (hsa_attn_bwd_tile.h) reads Q, dO and the leaf K / V twice: once per query
+// block for dQ, once per key block for dK / dV.  Here the wavefront that walks a strip of four
+// query blocks also finishes dK / dV of the strip's own four leaf key blocks: while a query block's
+// operands are in registers, its contribution to each leaf key block it attends is evaluated in
+// the second orientation (S[query, key], the queries in the MFMA contraction) and added to that
+// key block's accumulators; a key block is complete once the query block after it has been done.
+// What a strip's key blocks collect from the neighbouring strips' queries (the query block after
+// the strip, and without the causal mask the one before it) is rebuilt from three pieces of saved
+// state instead of being exchanged: the neighbour's Q and dO rows, the forward's log-sum-exp of
+// those queries (P = exp2(logit - lse)) and delta = <dO, O> from the forward's output rows.
+// So every row of Q, dO, K, V is fetched once per strip plus one halo block in four (or two),
+// nothing leaves as a partial result except the rows of levels >= 6 (one fp32 row per strip and
+// level, summed by a small second launch), and there are no atomics.
+//
+// What it costs: a wavefront now carries the key blocks' accumulators on top of everything the
+// query pass holds.  Between iterations they rest in LDS (else the kernel spills 85 registers or
+// drops to one wavefront per SIMD), which still leaves no room to request the next block's rows
+// ahead; the pass moves 0.73 of the two passes' bytes but waits more between requests, and takes
+// 65 us against 56 us at B8 H8 N2048 D64 with the causal mask (same run, same inputs).  It is
+// therefore offered beside the two-pass backward, not in its place: for callers who would
+// rather spend less of the memory system than less time (a backward that overlaps other work).
+#pragma once
+
+#include "hsa_attn_bwd_tile.h"
+
+namespace hsa {
+
+// Wavefronts per SIMD the fused pass is compiled for.
+constexpr int bwd_fused_waves(int D, bool causal) { return (D <= 32 || (D <= 64 && causal)) ? 2 : 1; }
+
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D, CAUSAL))))
+attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
+    using BT = BwdTile<T, D>;
+    using M_ = Mma<T>;
+    constexpr int NBW = 1, SB = BWD_STRIP;
+    constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD, CPR = BT::CPR;
+    constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
+    constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
+    constexpr int LDS_SLOTS = 4;
+    const BwdTileParams &p = fp.t;
+    __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
+    __shared__ __align__(16) float carry_mem[BWD_WPB * 2 * D];
+    __shared__ __align__(16) float delta_mem[BWD_WPB * TILE_Q];
+    // dK^T / dV^T of the key blocks that wait for the next query block (one when causal, two
+    // otherwise) rest here between iterations, so that they hold no registers while a block's
+    // scores and dQ are worked out: [slot][dK, dV][NJ][lane] 16-byte pieces
+    constexpr int NPARK = CAUSAL ? 1 : 2;
+    __shared__ __align__(16) f32x4 park_mem[BWD_WPB * NPARK * 2 * NJ * 64];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * BWD_WPB + wave;
+    if (unit >= p.n_units) return;
+    BT bt;
+    bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
+    const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
+    float *carry = carry_mem + wave * 2 * D;
+    float *delta_lds = delta_mem + wave * TILE_Q;
+    f32x4 *park = park_mem + wave * NPARK * 2 * NJ * 64 + (threadIdx.x & 63);
+    auto park_put = [&](int slot, const f32x4 (&tk)[NJ], const f32x4 (&tv)[NJ]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            park[((slot * 2 + 0) * NJ + j) * 64] = tk[j];
+            park[((slot * 2 + 1) * NJ + j) * 64] = tv[j];
+        }
+    };
+    auto park_get = [&](int slot, f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            tk[j] = park[((slot * 2 + 0) * NJ + j) * 64];
+            tv[j] = park[((slot * 2 + 1) * NJ + j) * 64];
+        }
+    };
+
+    const int N = p.N, L = p.L, R = p.R, H = p.H;
+    const int NB = N / TILE_Q, NS = NB / SB;
+    const int h = unit % H;
+    const int strip = (unit / H) % NS;
+    const int b = unit / (H * NS);
+    const int blk0 = strip * SB;
+    const int qs = blk0 * TILE_Q;  // first query of the strip
+    const size_t rs = (size_t)H * D;
+    const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Ob = fp.out + ((size_t)b * N * H + h) * D + 8 * lchk;
+    const uint16_t *Kb = p.k + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    const uint16_t *Vb = p.v + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+
+    // ---- tree slot constants (same slot layout as the forward kernel) -------------------------
+    int t_lvl[NLD], t_add[NLD], t_xor[NLD], u_row[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) {
+        const int sl = i * RPI + lrow;
+        if (sl < 8) { t_lvl[i] = 1; t_add[i] = sl; t_xor[i] = 0; }
+        else if (sl < 12) { t_lvl[i] = 2; t_add[i] = sl - 8; t_xor[i] = 0; }
+        else if (sl < 14) { t_lvl[i] = 3; t_add[i] = sl - 12; t_xor[i] = 0; }
+        else { t_lvl[i] = 4 + (sl - 14); t_add[i] = 0; t_xor[i] = 1; }
+        const int ul = 6 + sl;
+        u_row[i] = ul < L ? level_offset(N, ul) + ((qs >> ul) ^ 1) : -1;
+    }
+    auto near_row = [&](int i, int q0) {
+        return t_lvl[i] < L ? level_offset(N, t_lvl[i]) + (((q0 >> t_lvl[i]) + t_add[i]) ^ t_xor[i]) : -1;
+    };
+    auto slot_level = [](int sl, int &pl) {
+        if (sl < 8) { pl = sl; return 1; }
+        if (sl < 12) { pl = sl - 8; return 2; }
+        if (sl < 14) { pl = sl - 12; return 3; }
+        pl = -1;
+        return 4 + (sl - 14);
+    };
+    float b1U[4], b2U[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ul1 = 6 + 4 * g + i;
+        b1U[i] = (ul1 < L && (!CAUSAL || ((qs >> ul1) & 1))) ? 0.f : NEG_INF;
+        const int ul2 = 6 + r16;
+        b2U[i] = (ul2 < L && (!CAUSAL || ((qs >> ul2) & 1))) ? 0.f : NEG_INF;
+    }
+
+    // ---- loads ------------------------------------------------------------------------------
+    auto load_block = [&](const uint16_t *base, int row0, u32x4_t (&dst)[NLD]) {
+        const uint16_t *ptr = base + (size_t)(row0 + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) dst[i] = *reinterpret_cast<const u32x4_t *>(ptr + (size_t)(i * RPI) * rs);
+    };
+    auto leaf_row0 = [&](int kb) {
+        kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
+        return kb * TILE_Q;
+    };
+    struct Stage {
+        u32x4_t q[NLD], g[NLD], k[NLD], v[NLD], kt[NLD], vt[NLD];
+    };
+    auto request = [&](Stage &sg, int blk) {
+        const int q0 = blk * TILE_Q;
+        load_block(Qb, q0, sg.q);
+        load_block(Gb, q0, sg.g);
+        const int row0 = leaf_row0(blk - NBW + NKL - 1);
+        load_block(Kb, row0, sg.k);
+        load_block(Vb, row0, sg.v);
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int tr = near_row(i, q0);
+            sg.kt[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(tr < 0 ? q0 : tr) * rs);
+            sg.vt[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(tr < 0 ? q0 : tr) * rs);
+        }
+    };
+    // a neighbouring strip's query block: rows of Q, dO and of the forward's output, and the
+    // forward's log-sum-exp of its queries (4g + i)
+    struct Halo {
+        u32x4_t q[NLD], g[NLD], o[NLD];
+        float lse4[4];
+    };
+    auto request_halo = [&](Halo &hl, int qb) {
+        qb = qb < 0 ? 0 : (qb >= NB ? NB - 1 : qb);
+        load_block(Qb, qb * TILE_Q, hl.q);
+        load_block(Gb, qb * TILE_Q, hl.g);
+        load_block(Ob, qb * TILE_Q, hl.o);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) hl.lse4[i] = fp.lse[((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h];
+    };
+
+    // contribution of one query block (operands Qf/Gf, their transposes, the queries' lse and
+    // delta in the "regs = queries 4g+i" form) to the leaf key block kb (operands Kf/Vf)
+    auto leaf_contrib = [&](const u32x4_t (&Qf)[KS], const u32x4_t (&Gf)[KS], const u32x2_t (&QT)[NJ],
+                            const u32x2_t (&GT)[NJ], const float (&lse4)[4], const float (&del4)[4],
+                            const u32x4_t (&Kf)[KS], const u32x4_t (&Vf)[KS], int qb, int kb, f32x4 (&tk)[NJ],
+                            f32x4 (&tv)[NJ]) {
+        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            a = M_::k32(Qf[ks], Kf[ks], a);  // S[query 4g+i of block qb, key r16 of block kb]
+            d = M_::k32(Gf[ks], Vf[ks], d);
+        }
+        float pp[4], ds[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int ql = 4 * g + i;
+            const int diff = (kb - qb) * TILE_Q + r16 - ql;  // key - query
+            const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+            const bool sib = qb == kb && r16 == (ql ^ 1) && (!CAUSAL || (ql & 1));
+            const int cnt = (int)win + (int)sib;
+            const float bias = cnt == 0 ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+            pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
+            ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
+        }
+        const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+        const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            tk[j] = M_::k16(QT[j], dk, tk[j]);
+            tv[j] = M_::k16(GT[j], pk, tv[j]);
+        }
+    };
+    // contribution of a neighbouring strip's query block to one of this strip's key blocks
+    auto halo_contrib = [&](const Halo &hl, int qb, const u32x4_t (&Kf)[KS], const u32x4_t (&Vf)[KS], int kb,
+                            f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
+        // delta[q] = <dO[q], O[q]>: the lanes that share a row sum their pieces
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t gw = hl.g[i][w], ow = hl.o[i][w];
+                s = fmaf(to_float<T>((uint16_t)(gw & 0xffffu)), to_float<T>((uint16_t)(ow & 0xffffu)), s);
+                s = fmaf(to_float<T>((uint16_t)(gw >> 16)), to_float<T>((uint16_t)(ow >> 16)), s);
+            }
+#pragma unroll
+            for (int m = 1; m < CPR; m <<= 1) s += __shfl_xor(s, m, 64);
+            if (lchk == 0) delta_lds[i * RPI + lrow] = s;
+        }
+        u32x4_t Qf[KS], Gf[KS];
+        u32x2_t QT[NJ], GT[NJ];
+        bt.put(0, hl.q);
+        bt.put(1, hl.g);
+        bt.get(0, Qf);
+        bt.get(1, Gf);
+        bt.transpose(Qf, QT);
+        bt.transpose(Gf, GT);
+        float del4[4];
+        const f32x4 dl = *reinterpret_cast<const f32x4 *>(delta_lds + 4 * g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) del4[i] = dl[i];
+        leaf_contrib(Qf, Gf, QT, GT, hl.lse4, del4, Kf, Vf, qb, kb, tk, tv);
+    };
+    auto store_key_block = [&](int kb, const f32x4 (&tk)[NJ], const f32x4 (&tv)[NJ]) {
+        bt.put_result(0, tk, 1.0f);
+        bt.put_result(1, tv, 1.0f);
+        uint16_t *dKp = dKb + (size_t)(kb * TILE_Q + lrow) * rs;
+        uint16_t *dVp = dVb + (size_t)(kb * TILE_Q + lrow) * rs;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            *reinterpret_cast<u32x4_t *>(dKp + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
+            *reinterpret_cast<u32x4_t *>(dVp + (size_t)(i * RPI) * rs) = bt.get_row_piece(1, i);
+        }
+    };
+
+    // everything the first block needs is requested before anything is consumed
+    u32x4_t Kc[NKB][KS], Vc[NKB][KS];
+    Stage sg;
+    Halo halo;
+    const bool left_halo = !CAUSAL && blk0 > 0, right_halo = blk0 + SB < NB;  // uniform
+    {
+        u32x4_t rKu[NLD], rVu[NLD], rKh[NKL][NLD], rVh[NKL][NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            rKu[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
+            rVu[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
+        }
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+            load_block(Kb, leaf_row0(blk0 - NBW + c), rKh[c]);
+            load_block(Vb, leaf_row0(blk0 - NBW + c), rVh[c]);
+        }
+        if constexpr (!CAUSAL) request_halo(halo, blk0 - 1);
+        request(sg, blk0);
+        bt.put(2, rKu);
+        bt.put(3, rVu);
+        bt.get(2, Kc[NKL + 1]);
+        bt.get(3, Vc[NKL + 1]);
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+            bt.put(2, rKh[c]);
+            bt.put(3, rVh[c]);
+            bt.get(2, Kc[c]);
+            bt.get(3, Vc[c]);
+        }
+    }
+    if constexpr (!CAUSAL) {
+        // the query block before the strip reaches the strip's first key block (leaf block blk0,
+        // already here as the second carried-in block)
+        f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        if (left_halo) halo_contrib(halo, blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
+        park_put(0, tk, tv);
+    }
+    // partial rows of the far block, summed over the strip
+    f32x4 fk[NJ], fv[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+
+#pragma unroll
+    for (int it = 0; it < SB; ++it) {
+        const int blk = blk0 + it;
+        const int q0 = blk * TILE_Q;
+        if (it > 0) request(sg, blk);
+        u32x4_t Qf[KS], Gf[KS];
+        bt.put(0, sg.q);
+        bt.put(1, sg.g);
+        bt.put(2, sg.k);
+        bt.put(3, sg.v);
+        bt.get(0, Qf);
+        bt.get(1, Gf);
+        bt.get(2, Kc[NKL - 1]);
+        bt.get(3, Vc[NKL - 1]);
+        bt.put(2, sg.kt);
+        bt.put(3, sg.vt);
+        bt.get(2, Kc[NKL]);
+        bt.get(3, Vc[NKL]);
+
+        int t_row[NLD];
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) t_row[i] = near_row(i, q0);
+        float b1T[4], b2T[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            {
+                int pl;
+                const int lvl = slot_level(4 * g + i, pl);
+                const bool live = pl >= 0 ? (pl == ((r16 >> lvl) ^ 1) && (!CAUSAL || ((r16 >> lvl) & 1)))
+                                          : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+                b1T[i] = live ? 0.f : NEG_INF;
+            }
+            {
+                int pl;
+                const int lvl = slot_level(r16, pl);
+                const int ql = 4 * g + i;
+                const bool live = pl >= 0 ? (pl == ((ql >> lvl) ^ 1) && (!CAUSAL || ((ql >> lvl) & 1)))
+                                          : (lvl < L && (!CAUSAL || ((q0 >> lvl) & 1)));
+                b2T[i] = live ? 0.f : NEG_INF;
+            }
+        }
+        float biasL[NKL][4];
+#pragma unroll
+        for (int c = 0; c < NKL; ++c) {
+            const int dlt = TILE_Q * (c - NBW);
+            const int kb = blk - NBW + c;
+            const bool inside = kb >= 0 && kb < NB;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int kl = 4 * g + i;
+                const int diff = dlt + kl - r16;
+                const bool win = diff >= -R && diff <= (CAUSAL ? 0 : R);
+                const bool sib = dlt == 0 && kl == (r16 ^ 1) && (!CAUSAL || (r16 & 1));
+                const int cnt = (int)win + (int)sib;
+                biasL[c][i] = (!inside || cnt == 0) ? NEG_INF : (cnt == 2 ? 1.0f : 0.0f);
+            }
+        }
+
+        // ---- orientation 1: S^T, dP^T [key, query] ---------------------------------------------------
+        float sc[NKB][4], dp[NKB][4];
+        float mx = NEG_INF;
+#pragma unroll
+        for (int c = 0; c < NKB; ++c) {
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                a = M_::k32(Kc[c][ks], Qf[ks], a);
+                d = M_::k32(Vc[c][ks], Gf[ks], d);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
+                sc[c][i] = fmaf(a[i], p.scale_log2e, bias);
+                dp[c][i] = d[i];
+                mx = fmaxf(mx, sc[c][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float den = 0.f;
+#pragma unroll
+        for (int c = 0; c < NKB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[c][i] = __builtin_amdgcn_exp2f(sc[c][i] - mx);
+                den += sc[c][i];
+            }
+        den += __shfl_xor(den, 16, 64);
+        den += __shfl_xor(den, 32, 64);
+        const float inv = 1.0f / den;
+        float delta = 0.f;
+#pragma unroll
+        for (int c = 0; c < NKB; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                sc[c][i] *= inv;  // P
+                delta = fmaf(sc[c][i], dp[c][i], delta);
+            }
+        delta += __shfl_xor(delta, 16, 64);
+        delta += __shfl_xor(delta, 32, 64);
+        const float lse = mx + __builtin_amdgcn_logf(den);  // log2 domain: P = exp2(s' - lse)
+
+        // ---- dQ^T = sum_c K_c^T . dS_c^T ---------------------------------------------------------------
+        {
+            f32x4 acc[NJ];
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NKB; ++c) {
+                u32x2_t KT[NJ];
+                bt.transpose(Kc[c], KT);
+                float ds[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) ds[i] = sc[c][i] * (dp[c][i] - delta) * p.scale;
+                const u32x2_t dsp = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) acc[j] = M_::k16(KT[j], dsp, acc[j]);
+            }
+            bt.put_result(0, acc, 1.0f);
+            uint16_t *optr = p.dq + ((size_t)b * N * H + h) * D + 8 * lchk + (size_t)(q0 + lrow) * rs;
+#pragma unroll
+            for (int i = 0; i < NLD; ++i)
+                *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
+        }
+
+        // ---- orientation 2: dK^T, dV^T [channel, key] ---------------------------------------------------
+        u32x2_t QT[NJ], GT[NJ];
+        bt.transpose(Qf, QT);
+        bt.transpose(Gf, GT);
+        float lse4[4], del4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lse4[i] = __shfl(lse, 4 * g + i, 64);
+            del4[i] = __shfl(delta, 4 * g + i, 64);
+        }
+        if (it == SB - 1) request_halo(halo, blk0 + SB);  // arrives while the rest of the last block is computed
+        // the strip's own leaf key blocks this query block reaches, oldest first: the block before
+        // the query block is complete afterwards and leaves; the others rest in LDS
+#pragma unroll
+        for (int c = 0; c < NKL; ++c) {
+            const int j = it - NBW + c;  // key block within the strip
+            if (j >= 0 && j < SB) {
+                f32x4 tk[NJ], tv[NJ];
+                const bool fresh = c == NKL - 1 && (CAUSAL || j > 0);  // nobody has contributed yet
+                if (fresh) {
+#pragma unroll
+                    for (int jj = 0; jj < NJ; ++jj) { tk[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+                } else {
+                    park_get(j % NPARK, tk, tv);
+                }
+                leaf_contrib(Qf, Gf, QT, GT, lse4, del4, Kc[c], Vc[c], blk, blk0 + j, tk, tv);
+                if (c == 0) store_key_block(blk0 + j, tk, tv);
+                else park_put(j % NPARK, tk, tv);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int c = NKL + t;
+            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                a = M_::k32(Qf[ks], Kc[c][ks], a);   // S[query 4g+i, slot r16]
+                d = M_::k32(Gf[ks], Vc[c][ks], d);   // dP[query, slot]
+            }
+            float pp[4], ds[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float bias = t == 0 ? b2T[i] : b2U[i];
+                pp[i] = __builtin_amdgcn_exp2f(fmaf(a[i], p.scale_log2e, bias) - lse4[i]);
+                ds[i] = pp[i] * (d[i] - del4[i]) * p.scale;
+            }
+            const u32x2_t pk = u32x2_t{M_::pack(pp[0], pp[1]), M_::pack(pp[2], pp[3])};
+            const u32x2_t dk = u32x2_t{M_::pack(ds[0], ds[1]), M_::pack(ds[2], ds[3])};
+            if (t == 0) {
+                f32x4 tk[NJ], tv[NJ];
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+                    tk[j] = M_::k16(QT[j], dk, z);
+                    tv[j] = M_::k16(GT[j], pk, z);
+                }
+                // a level-5 node collects from the two blocks under its sibling, both this
+                // wavefront's: the even block parks its row, the odd block adds it: final
+                if (r16 == 15) {
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                        if (it & 1) {
+                            const f32x4 ck = *reinterpret_cast<const f32x4 *>(carry + ch);
+                            const f32x4 cv = *reinterpret_cast<const f32x4 *>(carry + D + ch);
+                            tk[j] += ck;
+                            tv[j] += cv;
+                        } else {
+                            *reinterpret_cast<f32x4 *>(carry + ch) = tk[j];
+                            *reinterpret_cast<f32x4 *>(carry + D + ch) = tv[j];
+                        }
+                    }
+                }
+                const bool five_final = (it & 1) != 0;
+                bt.put_result(0, tk, 1.0f);
+                bt.put_result(1, tv, 1.0f);
+#pragma unroll
+                for (int i = 0; i < NLD; ++i) {
+                    const int sl = i * RPI + lrow;
+                    if ((sl < 15 || five_final) && t_row[i] >= 0) {
+                        *reinterpret_cast<u32x4_t *>(dKb + (size_t)t_row[i] * rs) = bt.get_row_piece(0, i);
+                        *reinterpret_cast<u32x4_t *>(dVb + (size_t)t_row[i] * rs) = bt.get_row_piece(1, i);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    fk[j] = M_::k16(QT[j], dk, fk[j]);
+                    fv[j] = M_::k16(GT[j], pk, fv[j]);
+                }
+            }
+        }
+
+        // slide the leaf window by one block
+#pragma unroll
+        for (int c = 0; c + 1 < NKL; ++c) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) { Kc[c][ks] = Kc[c + 1][ks]; Vc[c][ks] = Vc[c + 1][ks]; }
+        }
+    }
+
+    // the strip's last key block: the query block after the strip reaches it (the block sits in
+    // the first operand slot after the last slide)
+    {
+        f32x4 tk[NJ], tv[NJ];
+        park_get((SB - 1) % NPARK, tk, tv);
+        if (right_halo) halo_contrib(halo, blk0 + SB, Kc[0], Vc[0], blk0 + SB - 1, tk, tv);
+        store_key_block(blk0 + SB - 1, tk, tv);
+    }
+
+    // levels >= 6: the strip's partial rows
+    {
+        const int lvl = 6 + r16;
+        const int LF = L - 6;
+        if (lvl < L) {
+            float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
+            const size_t po = ((((size_t)b * NS + strip) * H + h) * LF + (lvl - 6)) * D;
+            float *pkp = far + po;
+            float *pvp = far + (size_t)p.B * NS * H * LF * D + po;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
+                *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
+            }
+        }
+    }
+}
+
+// the rows of levels >= 6 (and the root row, the rows nobody attends, the rows past 2N-1) from the
+// strips' partial rows
+template <typename T>
+__global__ void __launch_bounds__(BWD_WPB * 64) attn_bwd_reduce_kernel(BwdTileParams p, int D) {
+    using S = typename T::storage;
+    bwd_reduce_rows<T>(p.partial, reinterpret_cast<S *>(p.dk), reinterpret_cast<S *>(p.dv), p.B, p.N, p.M, p.H, D, p.L,
+                       p.causal, p.red_first_row, p.red_lg_sb, (size_t)blockIdx.x * (BWD_WPB * 64) + threadIdx.x);
+}
+
+template <typename T, int D>
+int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
+
+#define HSA_BWD_FUSED_INSTANTIATE(T, D)                                                                     \
+    template <>                                                                                             \
+    int attn_bwd_fused_launch_td<T, D>(const BwdFusedParams &fp, bool causal, hipStream_t st) {             \
+        BwdFusedParams q = fp;                                                                              \
+        q.t.n_units = fp.t.n_units / BWD_STRIP;                                                             \
+        q.t.red_lg_sb = 2;                                                                                  \
+        const int nwg = (q.t.n_units + BWD_WPB - 1) / BWD_WPB;                                              \
+        if (causal) attn_bwd_tile_fused_kernel<T, D, true><<<nwg, BWD_WPB * 64, 0, st>>>(q);                \
+        else attn_bwd_tile_fused_kernel<T, D, false><<<nwg, BWD_WPB * 64, 0, st>>>(q);                      \
+        int rc = check_launch("attn_bwd_tile_fused_kernel");                                                \
+        if (rc != HSA_OK || q.t.red_wgs == 0) return rc;                                                    \
+        attn_bwd_reduce_kernel<T><<<q.t.red_wgs, BWD_WPB * 64, 0, st>>>(q.t, D);                            \
+        return check_launch("attn_bwd_reduce_kernel");                                                      \
+    }
+
+}  // namespace hsa

@@ -41,6 +41,13 @@ struct BwdTileParams {
     int causal, red_first_row, red_wgs, red_lg_sb;  // red_lg_sb: log2 of the query pass's blocks per strip
 };
 
+// the one-pass variant (hsa_attn_bwd_fused.h) also takes what the forward left behind
+struct BwdFusedParams {
+    BwdTileParams t;
+    const uint16_t *out;  // forward output [B, N, H, D]
+    const float *lse;     // forward log-sum-exp [B, N, H], log2 domain
+};
+
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
 
 // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; with this remap workgroups that

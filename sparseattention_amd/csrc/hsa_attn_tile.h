@@ -67,6 +67,7 @@ struct TileParams {
     const uint16_t *q, *k, *v;
     uint16_t *out;
     float *weights;  // [B, N, H, 2R+1+L] or null (kernels built with WT only)
+    float *lse;      // [B, N, H] or null: log-sum-exp of a query's biased logits, log2 domain
     int B, N, M, H, L, R;
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
@@ -425,6 +426,10 @@ attn_tile_kernel(TileParams p) {
         den += __shfl_xor(den, 16, 64);
         den += __shfl_xor(den, 32, 64);
         const float inv = 1.0f / den;
+        // what a backward pass needs to rebuild this query's weights without its whole row:
+        // P = exp2(logit * log2(e) / sqrt(D) + bias - lse)
+        if (p.lse != nullptr && g == 0)
+            p.lse[((size_t)b * p.N + q0 + r16) * p.H + h] = mx + __builtin_amdgcn_logf(den);
 
         if constexpr (WT) {
             // rows of weights in LDS: query r of the block at float offset r * S, in operand slots 1..4

@@ -66,7 +66,7 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
     return nbw <= TILE_MAX_NBW || (nbw <= TILE_MAX_NBW_WIDE && (D <= 64 || !want_weights));
 }
 
-int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, int B,
+int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, float *lse, int B,
                        int N, int M, int H, int D, int L, int R, int causal, int dtype, hipStream_t st) {
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
         return fail(HSA_ERR_INVALID, "tile kernel needs 16-byte aligned tensors");
@@ -74,6 +74,7 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v;
     p.out = (uint16_t *)out;
     p.weights = weights;
+    p.lse = lse;
     p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
     const int NB = N / TILE_Q;
     TileKnobs &knobs = tile_knobs();

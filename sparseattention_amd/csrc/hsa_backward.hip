@@ -735,6 +735,56 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
                    : attn_bwd_tile_launch_td<T, 128>(p, nbw, causal != 0, sb, st);
 }
 
+// ---- one-pass backward on saved forward state (hsa_attn_bwd_fused.h) ---------------------------
+template <typename T, int D>
+int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
+
+static bool attn_bwd_fused_eligible(int N, int M, int D, int L, int R, int dtype) {
+    if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
+    if (D != 32 && D != 64) return false;
+    if (N < TILE_Q * BWD_STRIP || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
+    return R <= TILE_Q;
+}
+// partial rows of dK and dV for levels >= 6, laid out like the two-pass workspace without its
+// statistics
+static size_t bwd_fused_ws_floats(int B, int N, int H, int D, int L) {
+    const size_t lv = 2 + (L > 6 ? L - 6 : 0);
+    return 2 * (size_t)B * (N / TILE_Q) * H * lv * D;
+}
+
+template <typename T>
+static int attn_bwd_fused_typed(const void *q, const void *k, const void *v, const void *out, const float *lse,
+                                const void *dout, void *dq, void *dk, void *dv, float *ws, int B, int N, int M,
+                                int H, int D, int L, int R, int causal, hipStream_t st) {
+    BwdFusedParams fp;
+    BwdTileParams &p = fp.t;
+    p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v; p.dout = (const uint16_t *)dout;
+    p.dq = (uint16_t *)dq; p.dk = (uint16_t *)dk; p.dv = (uint16_t *)dv;
+    p.stats = nullptr;
+    p.partial = ws;
+    fp.out = (const uint16_t *)out;
+    fp.lse = lse;
+    p.B = B; p.N = N; p.M = M; p.H = H; p.L = L; p.R = R;
+    const long units = (long)B * (N / TILE_Q) * H;
+    if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.n_units = (int)units;
+    p.scale = 1.0f / sqrtf((float)D);
+    p.scale_log2e = 1.4426950408889634f * p.scale;
+    // the strips finish levels 1..5; the rows above them, the root row and the rows past 2N-1 are
+    // summed from the strips' partial rows by a second, small launch
+    int first = level_offset(N, 6);
+    if (first > 2 * N - 2) first = 2 * N - 2;
+    const size_t red_threads = (size_t)B * (M - first) * H * (D / 4);
+    const size_t red_wgs = (red_threads + BWD_WPB * 64 - 1) / (BWD_WPB * 64);
+    if (red_wgs > 0x3fffffffUL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
+    p.causal = causal != 0;
+    p.red_first_row = first;
+    p.red_wgs = (int)red_wgs;
+    p.red_lg_sb = 2;
+    return D == 32 ? attn_bwd_fused_launch_td<T, 32>(fp, causal != 0, st)
+                   : attn_bwd_fused_launch_td<T, 64>(fp, causal != 0, st);
+}
+
 }  // namespace hsa
 
 extern "C" {
@@ -831,6 +881,35 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
         case HSA_BF16: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
     }
     return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype) {
+    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype)) return 0;
+    return hsa::bwd_fused_ws_floats(B, N, H, D, L) * sizeof(float);
+}
+
+int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *out, const float *lse,
+                       const void *dout, void *dq, void *dk, void *dv, void *workspace, size_t workspace_bytes, int B,
+                       int N, int M, int H, int D, int L, int R, int causal, int dtype, void *stream) {
+    HSA_REQUIRE(q && k && v && out && lse && dout && dq && dk && dv && workspace, "null pointer");
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
+    HSA_REQUIRE(hsa::ilog2_exact(N) == L, "canonical table needs L == log2 N (N=%d L=%d)", N, L);
+    HSA_REQUIRE(M >= 2 * N - 1, "canonical table needs M >= 2N-1 (N=%d M=%d)", N, M);
+    HSA_REQUIRE(R >= 0, "bad R=%d", R);
+    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward not available for N=%d D=%d L=%d R=%d dtype=%d "
+                         "(16-bit types, 32 or 64 channels per head, radius up to 16, at least 64 leaves)", N, D, L, R, dtype);
+    const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout |
+                           (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)workspace) & 15) == 0;
+    if (!aligned) return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward needs 16-byte aligned tensors");
+    HSA_REQUIRE(workspace_bytes >= hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, dtype),
+                "workspace too small (%zu bytes)", workspace_bytes);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == HSA_BF16)
+        return hsa::attn_bwd_fused_typed<hsa::BF16>(q, k, v, out, lse, dout, dq, dk, dv, (float *)workspace, B, N, M, H,
+                                                    D, L, R, causal, st);
+    return hsa::attn_bwd_fused_typed<hsa::F16>(q, k, v, out, lse, dout, dq, dk, dv, (float *)workspace, B, N, M, H, D,
+                                               L, R, causal, st);
 }
 
 // ---- hsa_attn_bwd for callers that must not allocate ---------------------------------------------

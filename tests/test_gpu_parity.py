@@ -1087,6 +1087,85 @@ def test_attention_backward_wide_causal_window_on_the_tile_passes(dtype):
         assert torch.equal(a, b)
 
 
+SAVED_BWD_CASES = [(2, 64, 2, 64, 16), (1, 128, 3, 64, 5), (2, 256, 4, 32, 16), (1, 512, 2, 64, 0), (2, 1024, 8, 64, 16),
+                   (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1)]
+
+
+@pytest.mark.parametrize("case", SAVED_BWD_CASES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_backward_from_saved_forward_state(case, causal, dtype):
+    """The one-pass backward (hsa_attn_bwd_saved) on the forward's output and log-sum-exp
+    (hsa_attn_fwd_lse): gradients against autograd through the fp64 oracle and against the
+    two-pass backward, the forward's output against the plain forward (bit for bit), and the
+    log-sum-exp against the oracle's logits.  One strip (no neighbours), first / last strips and
+    inner strips all occur."""
+    B, N, H, D, R = case
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=5 * N + R)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(N + R)).to(dtype)
+    o = oracle.topology_tables(N, causal)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    want_out, want_w = oracle.attention_ref(qr, kr, vr, o["forward_idx"], o["forward_mask"] if causal else None, R,
+                                            return_weights=True)
+    want_out.backward(go.double())
+    qd, kd, vd, gd = q.to(DEV), k.to(DEV), v.to(DEV), go.to(DEV)
+    assert fn.saved_state_backward_available(qd, kd, R)
+    out, lse = fn.attention_forward_lse(qd, kd, vd, R, causal)
+    t = sa.build_tree_topology(N, causal, device=DEV)
+    plain = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"] if causal else None, R)
+    assert torch.equal(out, plain)
+    # lse: log2 of the sum over slots of 2^(logit * log2(e) / sqrt(D)), the sibling leaf counted twice
+    L = N.bit_length() - 1
+    idx = torch.as_tensor(o["forward_idx"]).long()
+    n = torch.arange(N)
+    sc = torch.full((B, N, H, 2 * R + 1 + L), float("-inf"), dtype=torch.float64)
+    for w in range(2 * R + 1):
+        j = n + w - R
+        ok = (j >= 0) & (j < N) & ((j <= n) if causal else torch.ones_like(j, dtype=torch.bool))
+        jj = j.clamp(0, N - 1)
+        s = torch.einsum("bnhd,bnhd->bnh", q.double(), k.double()[:, jj]) / math.sqrt(D)
+        sc[..., w] = torch.where(ok[None, :, None], s, torch.full_like(s, float("-inf")))
+    for l in range(L):
+        live = ~torch.as_tensor(o["forward_mask"])[:, l] if causal else torch.ones(N, dtype=torch.bool)
+        s = torch.einsum("bnhd,bnhd->bnh", q.double(), k.double()[:, idx[:, l]]) / math.sqrt(D)
+        sc[..., 2 * R + 1 + l] = torch.where(live[None, :, None], s, torch.full_like(s, float("-inf")))
+    want_lse = torch.logsumexp(sc, dim=-1) / math.log(2.0)
+    assert (lse.double().cpu() - want_lse).abs().max() < 2e-2
+    got = fn.attention_backward_saved(gd, qd, kd, vd, out, lse, R, causal)
+    two = fn.attention_backward(gd, qd, kd, vd, R, causal)
+    for name, g1, g2, ref in zip(("dQ", "dK", "dV"), got, two, (qr.grad, kr.grad, vr.grad)):
+        _grad_close(g1, ref, dtype, "%s one pass, causal=%s" % (name, causal))
+        scale = max(1.0, float(ref.abs().max()))
+        assert (g1.float() - g2.float()).abs().max() <= 2e-2 * scale, "%s: one pass vs two passes" % name
+    # and through the autograd function: the two-pass backward unless the switch is on
+    for flag, ref in ((False, two), (True, got)):
+        qa, ka, va = (x.clone().requires_grad_(True) for x in (qd, kd, vd))
+        fn.one_pass_backward = flag
+        try:
+            sa.hierarchical_attention(qa, ka, va, t["forward_idx"], t["backward_gather"],
+                                      t["forward_mask"] if causal else None, R).backward(gd)
+        finally:
+            fn.one_pass_backward = False
+        for a, g1 in zip((qa.grad, ka.grad, va.grad), ref):
+            assert torch.equal(a, g1)
+
+
+def test_attention_backward_saved_state_limits():
+    """Shapes the one-pass backward does not take report it instead of launching."""
+    q = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, 127, 2, 64, dtype=torch.bfloat16, device=DEV)
+    assert fn.saved_state_backward_available(q, k, 16)
+    assert not fn.saved_state_backward_available(q, k, 17)                      # radius above one block
+    assert not fn.saved_state_backward_available(q.float(), k.float(), 16)      # fp32
+    assert not fn.saved_state_backward_available(q[:, :32], k[:, :63], 16)      # fewer than 64 leaves
+    q128 = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device=DEV)
+    assert not fn.saved_state_backward_available(q128, torch.zeros(1, 127, 2, 128, dtype=torch.bfloat16, device=DEV), 16)
+    lib = _lib.lib()
+    d = _lib.ptr(q)
+    rc = lib.hsa_attn_bwd_saved(d, d, d, d, d, d, d, d, d, d, 1 << 20, 1, 64, 127, 2, 64, 6, 17, 1, 2, _lib.stream_of(q))
+    assert rc == -95 and b"one-pass" in lib.hsa_last_error()
+
+
 WIDE_BWD_CASES = [(2, 512, 4, 64, 56), (1, 256, 2, 64, 33), (2, 128, 3, 32, 64), (1, 1024, 2, 32, 40),
                   (1, 32, 2, 64, 48), (1, 64, 1, 64, 64), (1, 16, 2, 32, 50), (1, 2048, 2, 64, 64)]
 
