@@ -570,6 +570,25 @@ def main():
     attn_bwd_ms = median(repeated(
         lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd(*bargs[i % nsets])), K, min_reps=7,
         min_total_ms=6.0))
+    # the one-pass backward on saved forward state (opt-in: less traffic, more time), where it applies
+    attn_bwd1_ms = None
+    if int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, _lib.HSA_BF16)) > 0:
+        saved = []
+        for s in prob.sets:
+            o_ = torch.empty_like(s["q"])
+            lse_ = torch.empty(B, N, H, device=dev, dtype=torch.float32)
+            assert lib.hsa_attn_fwd_lse(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), B, N, M, H, D, L, R,
+                                        int(causal), _lib.HSA_BF16, st) == 0, lib.hsa_last_error()
+            saved.append((o_, lse_))
+        b1args = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), P(gq), P(dq_), P(dk_), P(dv_), P(wsp),
+                   wsp.numel() * 4, B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, st)
+                  for s, (o_, lse_) in zip(prob.sets, saved)]
+        for i in range(3):
+            assert lib.hsa_attn_bwd_saved(*b1args[i % nsets]) == 0, lib.hsa_last_error()
+        attn_bwd1_ms = median(repeated(
+            lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd_saved(*b1args[i % nsets])), K,
+            min_reps=7, min_total_ms=6.0))
+        del saved, b1args
     del gq, dq_, dk_, dv_, wsp
 
     # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
@@ -629,6 +648,7 @@ def main():
                    "step_frac_of_hbm_peak_two_streams": step_algorithmic / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                    "attn_only_head_queries_per_s": head_queries / (attn_avg_ms * 1e-3),
                    "attn_backward_avg_ms": attn_bwd_ms,
+                   "attn_backward_one_pass_avg_ms": attn_bwd1_ms,
                    "attn_backward_algorithmic_bytes": E * B * H * D * (2 * N + 2 * M + N + 2 * M),
                    "device_copy_of_the_same_bytes": {
                        "bytes": copy_bytes, "avg_ms": copy_ms, "GBps": copy_bytes / (copy_ms * 1e-3) / 1e9,

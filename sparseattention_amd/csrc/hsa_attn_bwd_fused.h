@@ -17,11 +17,11 @@
 //
 // What it costs: a wavefront now carries the key blocks' accumulators on top of everything the
 // query pass holds.  Between iterations they rest in LDS (else the kernel spills 85 registers or
-// drops to one wavefront per SIMD), which still leaves no room to request the next block's rows
-// ahead; the pass moves 0.73 of the two passes' bytes but waits more between requests, and takes
-// 65 us against 56 us at B8 H8 N2048 D64 with the causal mask (same run, same inputs).  It is
-// therefore offered beside the two-pass backward, not in its place: for callers who would
-// rather spend less of the memory system than less time (a backward that overlaps other work).
+// drops to one wavefront per SIMD); 32 registers still spill, and there is no room to request the
+// next block's rows ahead.  Measured at B8 H8 N2048 D64 with the causal mask (rocprofv3, same run):
+// 261 MB of HBM traffic (scratch and halo rows included) against 283 MB for the two passes, 184.5 MB
+// algorithmic; 55.8 us + 5.6 us for the reduction against 32.0 + 18.5 us.  It is therefore offered
+// beside the two-pass backward, not in its place.
 #pragma once
 
 #include "hsa_attn_bwd_tile.h"

@@ -48,6 +48,9 @@ struct TreeArgs {
 
 constexpr int ilog2_const(int x) { return x <= 1 ? 0 : 1 + ilog2_const(x >> 1); }
 
+#ifndef TREE_DOT2
+#define TREE_DOT2 1
+#endif
 constexpr int TREE_NLMAX = 4;               // phase B: at most 16 subtrees per workgroup
 constexpr int TREE_GCAP_MAX = TREE_NLMAX + 2;  // phase C: at most 64 nodes per group
 
@@ -79,29 +82,85 @@ template <typename P> __device__ __forceinline__ P fetch_published(const void *s
     return *reinterpret_cast<const P *>(w);
 }
 
+// acc + <a, b> for two packed 16-bit elements with the two-element dot instruction: the products
+// are exact in fp32, the three-term sum is formed in fp32 (a level's dot products take a fifth of
+// the instructions of unpack + multiply-add; the levels of the launch's tail are bound by their
+// instruction count)
+template <typename T> __device__ __forceinline__ float dot2_acc(uint32_t a, uint32_t b, float acc);
+template <> __device__ __forceinline__ float dot2_acc<BF16>(uint32_t a, uint32_t b, float acc) {
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
+}
+template <> __device__ __forceinline__ float dot2_acc<F16>(uint32_t a, uint32_t b, float acc) {
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), acc, false);
+}
+
+// VEC floats -> a row piece, two elements per conversion where the type has a packed one
+template <typename T, int VEC> __device__ __forceinline__ VPack<T, VEC> pack_piece(const float (&o)[VEC]) {
+    VPack<T, VEC> r;
+    if constexpr (sizeof(typename T::storage) == 2 && VEC % 2 == 0) {
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        uint32_t *w = reinterpret_cast<uint32_t *>(&r);
+#pragma unroll
+        for (int i = 0; i < VEC / 2; ++i) {
+            const f32x2 v = {o[2 * i], o[2 * i + 1]};
+            if constexpr (T::id == HSA_BF16) {
+                typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+            } else {
+                typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+                w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) r.e[e] = from_float<T>(o[e]);
+    }
+    return r;
+}
+
+// the three scores of a parent: <q, k>, <q, c0>, <q, c1> over this lane's piece
+template <typename T, int VEC>
+__device__ __forceinline__ void scores3(const VPack<T, VEC> &q, const VPack<T, VEC> &k, const VPack<T, VEC> &c0,
+                                        const VPack<T, VEC> &c1, float &s0, float &s1, float &s2) {
+    s0 = 0.f; s1 = 0.f; s2 = 0.f;
+    if constexpr (sizeof(typename T::storage) == 2 && VEC % 2 == 0 && TREE_DOT2) {
+        const uint32_t *qw = reinterpret_cast<const uint32_t *>(&q), *kw = reinterpret_cast<const uint32_t *>(&k);
+        const uint32_t *aw = reinterpret_cast<const uint32_t *>(&c0), *bw = reinterpret_cast<const uint32_t *>(&c1);
+#pragma unroll
+        for (int w = 0; w < VEC / 2; ++w) {
+            s0 = dot2_acc<T>(qw[w], kw[w], s0);
+            s1 = dot2_acc<T>(qw[w], aw[w], s1);
+            s2 = dot2_acc<T>(qw[w], bw[w], s2);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float fq = to_float<T>(q.e[e]);
+            s0 = fmaf(fq, to_float<T>(k.e[e]), s0);
+            s1 = fmaf(fq, to_float<T>(c0.e[e]), s1);
+            s2 = fmaf(fq, to_float<T>(c1.e[e]), s2);
+        }
+    }
+}
+
 // one parent from its q/k/v row pieces and its two children's pieces (children are both key and value)
 template <typename T, int VEC>
 __device__ __forceinline__ VPack<T, VEC> combine(const VPack<T, VEC> &q, const VPack<T, VEC> &k,
                                                   const VPack<T, VEC> &v, const VPack<T, VEC> &c0,
                                                   const VPack<T, VEC> &c1, int G, float scale) {
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f;
-#pragma unroll
-    for (int e = 0; e < VEC; ++e) {
-        const float fq = to_float<T>(q.e[e]);
-        s0 = fmaf(fq, to_float<T>(k.e[e]), s0);
-        s1 = fmaf(fq, to_float<T>(c0.e[e]), s1);
-        s2 = fmaf(fq, to_float<T>(c1.e[e]), s2);
-    }
+    float s0, s1, s2;
+    scores3<T, VEC>(q, k, c0, c1, s0, s1, s2);
     s0 = group_sum(s0, G);
     s1 = group_sum(s1, G);
     s2 = group_sum(s2, G);
     float w0, w1, w2;
     softmax3<T>(s0 * scale, s1 * scale, s2 * scale, w0, w1, w2);
-    VPack<T, VEC> r;
+    float o[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e)
-        r.e[e] = from_float<T>(w0 * to_float<T>(v.e[e]) + w1 * to_float<T>(c0.e[e]) + w2 * to_float<T>(c1.e[e]));
-    return r;
+    for (int e = 0; e < VEC; ++e) o[e] = w0 * to_float<T>(v.e[e]) + w1 * to_float<T>(c0.e[e]) + w2 * to_float<T>(c1.e[e]);
+    return pack_piece<T, VEC>(o);
 }
 
 
@@ -237,23 +296,18 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
         // level 1: keys and values are different rows
 #pragma unroll
         for (int i = 0; i < NC / 2; ++i) {
-            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                const float fq = to_float<T>(rq[i].e[e]);
-                s0 = fmaf(fq, to_float<T>(rk[i].e[e]), s0);
-                s1 = fmaf(fq, to_float<T>(rck[2 * i].e[e]), s1);
-                s2 = fmaf(fq, to_float<T>(rck[2 * i + 1].e[e]), s2);
-            }
+            float s0, s1, s2;
+            scores3<T, VEC>(rq[i], rk[i], rck[2 * i], rck[2 * i + 1], s0, s1, s2);
             s0 = group_sum(s0, G);
             s1 = group_sum(s1, G);
             s2 = group_sum(s2, G);
             float w0, w1, w2;
             softmax3<T>(s0 * a.scale, s1 * a.scale, s2 * a.scale, w0, w1, w2);
+            float o[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
-                keep[i].e[e] = from_float<T>(w0 * to_float<T>(rv[i].e[e]) + w1 * to_float<T>(rcv[2 * i].e[e]) +
-                                             w2 * to_float<T>(rcv[2 * i + 1].e[e]));
+                o[e] = w0 * to_float<T>(rv[i].e[e]) + w1 * to_float<T>(rcv[2 * i].e[e]) + w2 * to_float<T>(rcv[2 * i + 1].e[e]);
+            keep[i] = pack_piece<T, VEC>(o);
             store_node<STREAM>(Out + node_row(1, sub * (NC / 2) + i), keep[i]);
         }
         // levels 2..TL

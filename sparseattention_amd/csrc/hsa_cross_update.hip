@@ -228,13 +228,15 @@ __device__ __forceinline__ void top_level(const TopParams &p, int b, int C, int 
 // flight, which is what bounds a wavefront that streams its head's weights from L2.  A level of
 // more than 16 children is shared out in 16-row tiles (blockIdx.z), each streaming the weights
 // again: the tiles run side by side instead of one wavefront multiplying them in turn.
-template <typename T, int CT2, int PD>
+// RT = 16-row tiles one wavefront multiplies side by side: with two, a level that would start more
+// wavefronts than the chip has SIMDs streams its weights half as often and runs in one round.
+template <typename T, int CT2, int PD, int RT = 1>
 __global__ void __launch_bounds__(64) cross_update_level_kernel(TopParams p, int C, int row, const uint16_t *lsrc,
                                                                 int64_t lsrc_bs, int64_t lsrc_rs) {
     const int b = blockIdx.x, h = blockIdx.y;
-    top_level_head<T, CT2, 1, false, PD>(p, b, h, C, row,
-                                         reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs), nullptr,
-                                         lsrc_rs * 2, (int)blockIdx.z);
+    top_level_head<T, CT2, RT, false, PD>(p, b, h, C, row,
+                                          reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs), nullptr,
+                                          lsrc_rs * 2, RT * (int)blockIdx.z);
 }
 
 template <typename T, int CT2, int RT0>
@@ -359,8 +361,16 @@ int top_launch_levels_pd(const TopParams &p, hipStream_t st) {
     const uint16_t *lsrc = p.src;
     int64_t lbs = p.src_bs, lrs = p.Dm;
     while (C >= 2) {
-        const dim3 grid((unsigned)p.B, (unsigned)p.H, (unsigned)((C + 15) / 16));
-        cross_update_level_kernel<T, CT2, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+        const int tiles = (C + 15) / 16;
+        // two row tiles per wavefront where single tiles would need a second round of wavefronts
+        // (1024 SIMDs; a lone wavefront's registers hold two tiles' operands up to 64 channels)
+        if (CT2 <= 4 && tiles % 2 == 0 && (long)p.B * p.H * tiles >= 2048) {
+            const dim3 grid((unsigned)p.B, (unsigned)p.H, (unsigned)(tiles / 2));
+            cross_update_level_kernel<T, CT2, PD, 2><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+        } else {
+            const dim3 grid((unsigned)p.B, (unsigned)p.H, (unsigned)tiles);
+            cross_update_level_kernel<T, CT2, PD><<<grid, 64, 0, st>>>(p, C, row, lsrc, lbs, lrs);
+        }
         // the next level's children are the rows just written
         lsrc = p.out + (size_t)row * p.out_rs;
         lbs = p.out_bs;
