@@ -15,13 +15,14 @@
 // nothing leaves as a partial result except the rows of levels >= 6 (one fp32 row per strip and
 // level, summed by a small second launch), and there are no atomics.
 //
-// What it costs: a wavefront now carries the key blocks' accumulators on top of everything the
-// query pass holds.  Between iterations they rest in LDS (else the kernel spills 85 registers or
-// drops to one wavefront per SIMD); 32 registers still spill, and there is no room to request the
-// next block's rows ahead.  Measured at B8 H8 N2048 D64 with the causal mask (rocprofv3, same run):
-// 261 MB of HBM traffic (scratch and halo rows included) against 283 MB for the two passes, 184.5 MB
-// algorithmic; 55.8 us + 5.6 us for the reduction against 32.0 + 18.5 us.  It is therefore offered
-// beside the two-pass backward, not in its place.
+// What it costs: a wavefront carries the waiting key blocks' accumulators on top of everything the
+// query pass holds: about 350 registers at 64 channels per head, i.e. one wavefront per SIMD
+// (two at 32 channels).  With two per SIMD it spilled (85 registers; 32 with the accumulators
+// resting in LDS between iterations) and took 65 us at B8 H8 N2048 D64 against 56 us for the two
+// passes; with one per SIMD, nothing spilled and the next block's rows requested one block ahead it
+// takes 56.0 us against 56.6 us (same run, inputs rotated through 1 GiB), 29.7 against 34.6 us at
+// B16 H8 N512, 104 against 113 us at B8 H8 N4096; without the causal mask and at 32 channels the
+// two passes stay 3-4 % ahead.
 #pragma once
 
 #include "hsa_attn_bwd_tile.h"
@@ -29,7 +30,7 @@
 namespace hsa {
 
 // Wavefronts per SIMD the fused pass is compiled for.
-constexpr int bwd_fused_waves(int D, bool causal) { return (D <= 32 || (D <= 64 && causal)) ? 2 : 1; }
+constexpr int bwd_fused_waves(int D, bool causal) { return D <= 32 ? 2 : 1; }
 
 template <typename T, int D, bool CAUSAL>
 __global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D, CAUSAL))))
@@ -45,11 +46,8 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
     __shared__ __align__(16) float carry_mem[BWD_WPB * 2 * D];
     __shared__ __align__(16) float delta_mem[BWD_WPB * TILE_Q];
-    // dK^T / dV^T of the key blocks that wait for the next query block (one when causal, two
-    // otherwise) rest here between iterations, so that they hold no registers while a block's
-    // scores and dQ are worked out: [slot][dK, dV][NJ][lane] 16-byte pieces
+    // dK^T / dV^T of the key blocks that wait for the next query block: one when causal, two otherwise
     constexpr int NPARK = CAUSAL ? 1 : 2;
-    __shared__ __align__(16) f32x4 park_mem[BWD_WPB * NPARK * 2 * NJ * 64];
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * BWD_WPB + wave;
@@ -59,21 +57,17 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
     float *carry = carry_mem + wave * 2 * D;
     float *delta_lds = delta_mem + wave * TILE_Q;
-    f32x4 *park = park_mem + wave * NPARK * 2 * NJ * 64 + (threadIdx.x & 63);
+    // slots are compile-time constants: plain registers
+    f32x4 PK[NPARK][NJ], PV[NPARK][NJ];
     auto park_put = [&](int slot, const f32x4 (&tk)[NJ], const f32x4 (&tv)[NJ]) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            park[((slot * 2 + 0) * NJ + j) * 64] = tk[j];
-            park[((slot * 2 + 1) * NJ + j) * 64] = tv[j];
-        }
+        for (int j = 0; j < NJ; ++j) { PK[slot][j] = tk[j]; PV[slot][j] = tv[j]; }
     };
     auto park_get = [&](int slot, f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
 #pragma unroll
-        for (int j = 0; j < NJ; ++j) {
-            tk[j] = park[((slot * 2 + 0) * NJ + j) * 64];
-            tv[j] = park[((slot * 2 + 1) * NJ + j) * 64];
-        }
+        for (int j = 0; j < NJ; ++j) { tk[j] = PK[slot][j]; tv[j] = PV[slot][j]; }
     };
+
 
     const int N = p.N, L = p.L, R = p.R, H = p.H;
     const int NB = N / TILE_Q, NS = NB / SB;
@@ -241,7 +235,8 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 
     // everything the first block needs is requested before anything is consumed
     u32x4_t Kc[NKB][KS], Vc[NKB][KS];
-    Stage sg;
+    Stage sgs[2];
+    Stage &sg = sgs[0];
     Halo halo;
     const bool left_halo = !CAUSAL && blk0 > 0, right_halo = blk0 + SB < NB;  // uniform
     {
@@ -288,7 +283,8 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     for (int it = 0; it < SB; ++it) {
         const int blk = blk0 + it;
         const int q0 = blk * TILE_Q;
-        if (it > 0) request(sg, blk);
+        Stage &sg = sgs[it & 1];
+        if (it + 1 < SB) request(sgs[(it + 1) & 1], blk + 1);  // the next block's rows, one block ahead
         u32x4_t Qf[KS], Gf[KS];
         bt.put(0, sg.q);
         bt.put(1, sg.g);

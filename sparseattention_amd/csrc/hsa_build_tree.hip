@@ -407,6 +407,35 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
         // ---- arrival: the last workgroup of a group to arrive continues upwards ----------------
         const int g = lg_width < gcap ? lg_width : gcap;
         const int grp = idx >> g;
+        // Where the closing workgroup will read: worked out by every workgroup before it waits
+        // for its stores, so that whoever closes the group has nothing left to do after the
+        // counter's answer but to request the rows.  The stage's first level takes its children
+        // (the group's published nodes) and parents from registers, maybe in two passes over the
+        // slots; the parents of the levels above go to LDS slots t and t + THREADS of the run that
+        // follows.  Slots and levels that do not exist re-read the nearest one.
+        const bool two = ((1 << (g - 1)) << lgH) > upb;
+        const int lgw = g - 1 + lgH + lgG;   // log2 of the next run's w1x2
+        size_t o_child[2], o_par[2], o_up[2];
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            const int p = (u_local + pass * upb) >> lgH;
+            const int np = 1 << (g - 1);
+            const int pc = p < np ? p : np - 1;
+            o_child[pass] = node_row(level, (grp << g) + 2 * pc);
+            o_par[pass] = node_row(level + 1, (grp << (g - 1)) + pc);
+            const int sl = (int)threadIdx.x + pass * THREADS;
+            const int m = (1 << lgw) - 1 - sl;
+            int jj = lgw - (31 - __clz((m > 0 ? m : 0) | 1));
+            jj = jj < g - 1 ? jj : g - 1;
+            jj = jj > 0 ? jj : 0;               // g == 1: no run; the stage's own parent row
+            const int first = jj > 0 ? (1 << lgw) - ((1 << lgw) >> (jj - 1)) : 0;
+            const int npu = 1 << (g - 1 - jj);
+            int pp = (sl - first) >> (lgH + lgG);
+            pp = pp < npu ? pp : npu - 1;
+            pp = pp > 0 ? pp : 0;
+            o_up[pass] = node_row(level + 1 + jj, (grp << (g - 1 - jj)) + pp);
+            asm volatile("" : "+v"(o_child[pass]), "+v"(o_par[pass]), "+v"(o_up[pass]));  // computed here, not after the wait
+        }
         // This workgroup's node has been written with device-scope (sc1) stores, which the L2
         // writes through to memory; such a store is acknowledged -- the wavefront's vmcnt drops --
         // only when the write has reached the memory side, the point where every XCD's L2 misses
@@ -432,47 +461,24 @@ __global__ void __launch_bounds__(THREADS) build_tree_fused_kernel(TreeArgs a) {
         }
         asm volatile("" ::: "memory");
 
-        // ---- the closing workgroup: the stage's first level from registers ----------------------
-        // Its children are the group's published nodes; it may take two passes over the slots.
-        // The parents of the levels above are requested together with them and staged in LDS for
-        // the run that follows.  All loads are unconditional: slots and levels that do not exist
-        // re-read the nearest one.
-        const bool two = ((1 << (g - 1)) << lgH) > upb;
+        // ---- the closing workgroup ---------------------------------------------------------------
         P cq[2], ckk[2], cvv[2], ch0[2], ch1[2];
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
         u4 uq[2], uk[2], uv[2];
-#pragma unroll
-        for (int pass = 0; pass < 2; ++pass) {
-            const int p = (u_local + pass * upb) >> lgH;
-            const int np = 1 << (g - 1);
-            const int pc = p < np ? p : np - 1;
-            const size_t crow = node_row(level, (grp << g) + 2 * pc);
-            ch0[pass] = fetch_published<P>(Out + crow);
-            ch1[pass] = fetch_published<P>(Out + crow + rs);
-            const size_t row = node_row(level + 1, (grp << (g - 1)) + pc);
-            cq[pass] = *reinterpret_cast<const P *>(Qp + row);
-            ckk[pass] = *reinterpret_cast<const P *>(Kp + row);
-            cvv[pass] = *reinterpret_cast<const P *>(Vp + row);
-        }
-        // staging slots t and t + THREADS of the run that follows (levels 2..g of the stage)
-        const int lgw = g - 1 + lgH + lgG;   // log2 of w1x2
         w1x2 = 1 << lgw;
 #pragma unroll
         for (int pass = 0; pass < 2; ++pass) {
-            const int sl = (int)threadIdx.x + pass * THREADS;
-            const int m = w1x2 - 1 - sl;
-            int jj = lgw - (31 - __clz((m > 0 ? m : 0) | 1));
-            jj = jj < g - 1 ? jj : g - 1;
-            jj = jj > 0 ? jj : 0;               // g == 1: no run; the stage's own parent row
-            const int first = jj > 0 ? w1x2 - (w1x2 >> (jj - 1)) : 0;
-            const int np = 1 << (g - 1 - jj);
-            int pp = (sl - first) >> (lgH + lgG);
-            pp = pp < np ? pp : np - 1;
-            pp = pp > 0 ? pp : 0;
-            const size_t row = node_row(level + 1 + jj, (grp << (g - 1 - jj)) + pp);
-            uq[pass] = *reinterpret_cast<const u4 *>(Qp + row);
-            uk[pass] = *reinterpret_cast<const u4 *>(Kp + row);
-            uv[pass] = *reinterpret_cast<const u4 *>(Vp + row);
+            ch0[pass] = fetch_published<P>(Out + o_child[pass]);
+            ch1[pass] = fetch_published<P>(Out + o_child[pass] + rs);
+            cq[pass] = *reinterpret_cast<const P *>(Qp + o_par[pass]);
+            ckk[pass] = *reinterpret_cast<const P *>(Kp + o_par[pass]);
+            cvv[pass] = *reinterpret_cast<const P *>(Vp + o_par[pass]);
+        }
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            uq[pass] = *reinterpret_cast<const u4 *>(Qp + o_up[pass]);
+            uk[pass] = *reinterpret_cast<const u4 *>(Kp + o_up[pass]);
+            uv[pass] = *reinterpret_cast<const u4 *>(Vp + o_up[pass]);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll

@@ -380,20 +380,30 @@ class BuildParentNodesFunc(torch.autograd.Function):
         return build_parents_backward(grad_output, *ctx.saved_tensors)
 
 
-# The backward of `hierarchical_attention` runs two passes over Q, dO and the leaf K / V by default
-# (the faster one: 50.5 us of kernel time against 61.4 us at B8 H8 N2048 D64).  With this switch on,
-# the forward also keeps its output and one log-sum-exp per (query, head), and the backward runs in
-# one pass where the shape allows (16-bit types, 32 / 64 channels per head, window radius up to
-# 16): 261 MB instead of 283 MB of memory traffic at that shape.  Process-wide; read when the
-# forward runs.
-one_pass_backward = False
+# Which backward `hierarchical_attention` uses.  Two formulations exist: two passes over Q, dO and
+# the leaf K / V (any shape the tile kernels take), and one pass that works from the forward's
+# output and one log-sum-exp per (query, head), which the forward then keeps (16-bit types, 32 / 64
+# channels per head, window radius up to 16).  The one pass moves less (0.86 of the two passes' HBM
+# traffic at B8 H8 N2048 D64) and is as fast or faster with the causal mask at 64 channels per head
+# (56.0 against 56.6 us there, 29.7 against 34.6 us at B16 H8 N512); without the mask and at 32
+# channels the two passes are 3-4 % ahead.
+#   None (default): the one pass where it measured at least as fast (causal, 64 channels per head)
+#   True / False:   the one pass wherever it applies / never
+# Process-wide; read when the forward runs.
+one_pass_backward = None
+
+
+def _use_one_pass(Q, K, window_size, causal) -> bool:
+    if one_pass_backward is False or not saved_state_backward_available(Q, K, window_size):
+        return False
+    return True if one_pass_backward else (bool(causal) and Q.shape[3] == 64)
 
 
 class HierarchicalAttentionFunc(torch.autograd.Function):
     """Forward + backward of the span attention (reference: HierarchicalAttentionFunc,
     hierarchical_attention/ops/functional.py:116-264, which keeps Q, K, V, the tables and its
-    Weights tensor for the backward).  Kept here: Q, K, V and, with `one_pass_backward`, the
-    output and one log-sum-exp per (query, head)."""
+    Weights tensor for the backward).  Kept here: Q, K, V and, where the one-pass backward is
+    used (`one_pass_backward`), the output and one log-sum-exp per (query, head)."""
 
     @staticmethod
     def forward(ctx, Q, K, V, idx_table, gather_table, mask_table=None, window_size=16):
@@ -406,8 +416,8 @@ class HierarchicalAttentionFunc(torch.autograd.Function):
         ctx.canonical = canon
         ctx.window_size = int(window_size)
         ctx.saved_state = False
-        if (one_pass_backward and canon is not None and K.shape[1] >= 2 * N - 1 and Q.dtype == K.dtype == V.dtype
-                and K.shape == V.shape and saved_state_backward_available(Q, K, window_size)):
+        if (canon is not None and K.shape[1] >= 2 * N - 1 and Q.dtype == K.dtype == V.dtype
+                and K.shape == V.shape and _use_one_pass(Q, K, window_size, canon)):
             res = attention_forward_lse(Q, K, V, window_size, canon)
             if res is not None:
                 out, lse = res
