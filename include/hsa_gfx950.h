@@ -317,8 +317,9 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
  * HSA_ERR_UNSUPPORTED (hsa_attn_bwd_saved_workspace_bytes returns 0) and the caller uses
  * hsa_attn_bwd.  workspace: hsa_attn_bwd_saved_workspace_bytes(...) bytes, written before read.
  *
- * hsa_attn_fwd_lse: hsa_attn_fwd on the canonical tables that also writes lse (16-bit tile kernel
- * only; HSA_ERR_UNSUPPORTED otherwise, nothing launched).
+ * hsa_attn_fwd_lse: hsa_attn_fwd on the canonical tables that also writes lse (a variant of the
+ * 16-bit tile kernel, built for the shapes hsa_attn_bwd_saved takes: up to 64 channels per head,
+ * window radius up to 16; HSA_ERR_UNSUPPORTED otherwise, nothing launched).
  */
 int hsa_attn_fwd_lse(const void *q, const void *k, const void *v, void *out, float *lse, int B, int N, int M,
                      int H, int D, int L, int R, int causal, int dtype, void *stream);

@@ -67,7 +67,7 @@ struct TileParams {
     const uint16_t *q, *k, *v;
     uint16_t *out;
     float *weights;  // [B, N, H, 2R+1+L] or null (kernels built with WT only)
-    float *lse;      // [B, N, H] or null: log-sum-exp of a query's biased logits, log2 domain
+    float *lse;      // [B, N, H]: log-sum-exp of a query's biased logits, log2 domain (kernels built with LSE only)
     int B, N, M, H, L, R;
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
@@ -94,7 +94,7 @@ template <int D, int NKL = 1> constexpr int tile_max_wpb() { return (D > 64 || N
 // dead slots zero).  A block's 16 rows of weights are assembled in the wavefront's LDS region
 // (the operand slots are free once the MFMA operands have been read) and written out as
 // whole rows.  Needs 2R+1+L <= D*2+16 floats per row to fit.
-template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false>
+template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false, bool LSE = false>
 __global__ void __launch_bounds__((tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>() * 64))
 attn_tile_kernel(TileParams p) {
     using M_ = Mma<T>;
@@ -428,8 +428,11 @@ attn_tile_kernel(TileParams p) {
         const float inv = 1.0f / den;
         // what a backward pass needs to rebuild this query's weights without its whole row:
         // P = exp2(logit * log2(e) / sqrt(D) + bias - lse)
-        if (p.lse != nullptr && g == 0)
-            p.lse[((size_t)b * p.N + q0 + r16) * p.H + h] = mx + __builtin_amdgcn_logf(den);
+        // (a variant of its own: as a run-time branch it cost the widest variants their last
+        // registers, B8 H8 N2048 D64 without the causal mask 20.4 -> 23.7 us)
+        if constexpr (LSE) {
+            if (g == 0) p.lse[((size_t)b * p.N + q0 + r16) * p.H + h] = mx + __builtin_amdgcn_logf(den);
+        }
 
         if constexpr (WT) {
             // rows of weights in LDS: query r of the block at float offset r * S, in operand slots 1..4
@@ -535,5 +538,7 @@ int attn_tile_launch_td(const TileParams &p, int nbw, bool causal, int sb, int w
 // the variant that also writes the softmax weights (one query block per wavefront)
 template <typename T, int D>
 int attn_tile_weights_launch_td(const TileParams &p, int nbw, bool causal, int wpb, hipStream_t st);
+template <typename T, int D>
+int attn_tile_lse_launch_td(const TileParams &p, int nbw, bool causal, int sb, int wpb, hipStream_t st);
 
 }  // namespace hsa

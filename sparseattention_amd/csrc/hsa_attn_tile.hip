@@ -126,6 +126,17 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
         if (D == 64) return attn_tile_weights_launch_td<F16, 64>(p, nbw, causal != 0, wpb, st);
         return attn_tile_weights_launch_td<F16, 128>(p, nbw, causal != 0, wpb, st);
     }
+    if (lse) {
+        if (weights) return fail(HSA_ERR_UNSUPPORTED, "weights and log-sum-exp outputs together are not built");
+        if (dtype == HSA_BF16) {
+            if (D == 32) return attn_tile_lse_launch_td<BF16, 32>(p, nbw, causal != 0, sb, wpb, st);
+            if (D == 64) return attn_tile_lse_launch_td<BF16, 64>(p, nbw, causal != 0, sb, wpb, st);
+            return attn_tile_lse_launch_td<BF16, 128>(p, nbw, causal != 0, sb, wpb, st);
+        }
+        if (D == 32) return attn_tile_lse_launch_td<F16, 32>(p, nbw, causal != 0, sb, wpb, st);
+        if (D == 64) return attn_tile_lse_launch_td<F16, 64>(p, nbw, causal != 0, sb, wpb, st);
+        return attn_tile_lse_launch_td<F16, 128>(p, nbw, causal != 0, sb, wpb, st);
+    }
     if (dtype == HSA_BF16) {
         if (D == 32) return attn_tile_launch_td<BF16, 32>(p, nbw, causal != 0, sb, wpb, st);
         if (D == 64) return attn_tile_launch_td<BF16, 64>(p, nbw, causal != 0, sb, wpb, st);

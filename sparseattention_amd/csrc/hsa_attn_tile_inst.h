@@ -21,6 +21,25 @@ static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
     return check_launch("attn_tile_kernel");
 }
 
+// the variant that also writes the queries' log-sum-exp (window radius up to 16, up to 64 channels)
+template <typename T, int D, int NBW, bool CAUSAL>
+static int tile_launch_lse(const TileParams &p, int sb, int wpb, hipStream_t st) {
+    if constexpr (D <= 64) {
+        constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
+        if (wpb > MAXW) wpb = MAXW;
+        const int nwg = (p.n_units + wpb - 1) / wpb;
+        switch (sb) {
+            case 1: attn_tile_kernel<T, D, NBW, CAUSAL, 1, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+            case 2: attn_tile_kernel<T, D, NBW, CAUSAL, 2, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+            case 4: attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+            default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
+        }
+        return check_launch("attn_tile_kernel (log-sum-exp)");
+    } else {
+        return fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output is built for up to 64 channels per head");
+    }
+}
+
 template <typename T, int D, int NBW, bool CAUSAL>
 static int tile_launch_weights(const TileParams &p, int wpb, hipStream_t st) {
     constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
@@ -71,6 +90,17 @@ static int tile_launch_wide_weights(const TileParams &p, int wpb, hipStream_t st
             case 9: return tile_launch_sb<T, D, 4, true>(p, sb, wpb, st);                       \
         }                                                                                       \
         return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel");       \
+    }                                                                                           \
+    template <>                                                                                 \
+    int attn_tile_lse_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int sb,       \
+                                      int wpb, hipStream_t st) {                                \
+        switch (nbw * 2 + (causal ? 1 : 0)) {                                                   \
+            case 0: return tile_launch_lse<T, D, 0, false>(p, sb, wpb, st);                     \
+            case 1: return tile_launch_lse<T, D, 0, true>(p, sb, wpb, st);                      \
+            case 2: return tile_launch_lse<T, D, 1, false>(p, sb, wpb, st);                     \
+            case 3: return tile_launch_lse<T, D, 1, true>(p, sb, wpb, st);                      \
+        }                                                                                       \
+        return fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output is built for window radius up to 16"); \
     }                                                                                           \
     template <>                                                                                 \
     int attn_tile_weights_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int wpb,  \
