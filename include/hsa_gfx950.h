@@ -67,8 +67,8 @@ const char *hsa_last_error(void);
  *   dtype       HSA_F32 / HSA_F16 / HSA_BF16
  *   algo        HSA_ATTN_*.  The MFMA tile kernels take canonical tables (idx == NULL),
  *               16 <= N <= 2^22, R <= 32 (16-bit types: R <= 64), head sizes 32 / 64 / 128, and
- *               write weights only for the 16-bit types (for 32 < R <= 64 without the causal mask
- *               only up to head size 64); everything else runs on the gather kernel
+ *               write weights only for the 16-bit types; everything else runs on the gather
+ *               kernel
  */
 int hsa_attn_fwd(const void *q, const void *k, const void *v, const int32_t *idx,
                  const uint8_t *mask, void *out, float *weights, int B, int N, int M, int H,
@@ -286,13 +286,10 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
  *   q, dout, dq  [B, N, H, D];  k, v, dk, dv  [B, M, H, D], M >= 2N-1
  *   workspace    device memory of at least hsa_attn_bwd_workspace_bytes(...) bytes, provided by
  *                the caller (scratch only: nothing in it has to survive the call)
- *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (16-bit: head size 32, 64 or 128,
- *                R <= 32, and R <= 64 with the causal mask or up to head size 64; fp32: head size
- *                32 or 64, R <= 32: a query-stationary pass and a key-stationary pass that also
- *                sums the first pass's fp32 partial rows for the upper tree levels), else the
- *                gather kernels; both are deterministic (no atomics).  The workspace query does
- *                not know whether the call will be causal: for 32 < R <= 64 at head size 128 it
- *                reports what either formulation needs.
+ *   algo         HSA_ATTN_AUTO: MFMA tile kernels when eligible (head size 32, 64 or 128; 16-bit:
+ *                R <= 64; fp32: R <= 32: a query-stationary pass and a key-stationary pass that
+ *                also sums the first pass's fp32 partial rows for the upper tree levels), else the
+ *                gather kernels; both are deterministic (no atomics).
  *                Tensors that are not 16-byte aligned run on the gather kernels and need the
  *                workspace size reported for HSA_ATTN_GATHER.
  */

@@ -105,8 +105,9 @@ __device__ __forceinline__ int near_slot_level(int sl, int &pl) {
 // (A) query pass
 // ---------------------------------------------------------------------------------------------
 // Wavefronts per SIMD the query pass is compiled for: two (256 registers) up to three leaf blocks
-// per query block, where at most a few words spill; one with five leaf blocks at D = 64.
-constexpr int f32b_query_waves(int D, int nkl) { return (D <= 32 || nkl <= 3) ? 2 : 1; }
+// per query block, where at most a few words spill; one with five leaf blocks at D = 64 and
+// always at D = 128 (there part of the operands lives in per-lane scratch memory).
+constexpr int f32b_query_waves(int D, int nkl) { return D >= 128 ? 1 : ((D <= 32 || nkl <= 3) ? 2 : 1); }
 
 template <int D, int NBW, bool CAUSAL>
 __global__ void __launch_bounds__(F32B_WPB * 64)
@@ -530,10 +531,10 @@ int launch_d(const BwdF32Params &p, int nbw, bool causal, hipStream_t st) {
 
 }  // namespace
 
-// fp32 tensors, head size 32 or 64, canonical tables, R <= 32 (at most five leaf blocks per query
-// block: all of a block's rows are in flight at once)
+// fp32 tensors, head size 32, 64 or 128, canonical tables, R <= 32 (at most five leaf blocks per
+// query block: all of a block's rows are in flight at once)
 bool attn_bwd_tile_f32_eligible(int N, int M, int D, int L, int R) {
-    if (D != 32 && D != 64) return false;
+    if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
     return R <= 2 * TILE_Q;
 }
@@ -565,7 +566,9 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
     p.causal = causal != 0;
     p.red_first_row = first;
     p.red_wgs = (int)red_wgs;
-    return D == 32 ? launch_d<32>(p, nbw, causal != 0, st) : launch_d<64>(p, nbw, causal != 0, st);
+    return D == 32 ? launch_d<32>(p, nbw, causal != 0, st)
+         : D == 64 ? launch_d<64>(p, nbw, causal != 0, st)
+                   : launch_d<128>(p, nbw, causal != 0, st);
 }
 
 }  // namespace hsa

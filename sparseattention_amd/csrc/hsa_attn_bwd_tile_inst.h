@@ -28,11 +28,16 @@ static int bwd_tile_launch_one(const BwdTileParams &p, int sb, hipStream_t st) {
 }
 
 // Windows of 33..64 neighbours to either side without the causal mask (seven or nine leaf blocks
-// per query block): head sizes up to 64 hold that many blocks in registers, one wavefront per SIMD.
+// per query block): head sizes up to 64 hold that many blocks in registers, one wavefront per SIMD;
+// at 128 channels only one block per wavefront is built (the caller passes sb = 1), and the key
+// pass keeps part of its operands in per-lane scratch memory.
 template <typename T, int D, int NBW>
 static int bwd_tile_launch_wide(const BwdTileParams &p, int sb, hipStream_t st) {
     if constexpr (D <= 64) return bwd_tile_launch_one<T, D, NBW, false>(p, sb, st);
-    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile backward at this head size");
+    else {
+        if (sb != 1) return fail(HSA_ERR_INVALID, "internal: strip length %d not built at this radius and head size", sb);
+        return bwd_tile_launch_sb<T, D, NBW, false, 1>(p, st);
+    }
 }
 
 template <typename T, int D>

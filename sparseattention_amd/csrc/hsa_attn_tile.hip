@@ -62,8 +62,8 @@ bool attn_tile_eligible(int N, int M, int H, int D, int L, int R, int dtype, boo
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     if (causal) return nbw <= TILE_MAX_NBW_CAUSAL;
     // without the causal mask: up to five leaf blocks everywhere, seven or nine with one query
-    // block per wavefront (the weights output only up to 64 channels per head)
-    return nbw <= TILE_MAX_NBW || (nbw <= TILE_MAX_NBW_WIDE && (D <= 64 || !want_weights));
+    // block per wavefront
+    return nbw <= TILE_MAX_NBW || nbw <= TILE_MAX_NBW_WIDE;
 }
 
 int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, float *weights, float *lse, int B,

@@ -66,11 +66,10 @@ template <typename T, int D, int NBW>
 static int tile_launch_wide(const TileParams &p, int wpb, hipStream_t st) {
     return tile_launch_one<T, D, NBW, false, 1>(p, wpb, st);
 }
-// the same with the weights output, head sizes up to 64
+// the same with the weights output
 template <typename T, int D, int NBW>
 static int tile_launch_wide_weights(const TileParams &p, int wpb, hipStream_t st) {
-    if constexpr (D <= 64) return tile_launch_weights<T, D, NBW, false>(p, wpb, st);
-    else return fail(HSA_ERR_UNSUPPORTED, "window radius too large for the tile kernel's weights at this head size");
+    return tile_launch_weights<T, D, NBW, false>(p, wpb, st);
 }
 
 #define HSA_TILE_INSTANTIATE(T, D)                                                              \

@@ -675,20 +675,15 @@ int attn_bwd_tile_f32_dispatch(const void *q, const void *k, const void *v, cons
                                void *dv, float *ws, int B, int N, int M, int H, int D, int L, int R, int causal,
                                hipStream_t st);
 
-// causal: 1 / 0, or -1 when the caller does not know yet (the workspace query): then "eligible
-// with the causal mask only" counts as eligible.  16-bit types take R <= 32, and R <= 64 with the
-// causal mask or with heads of at most 64 channels.
+// 16-bit types take R <= 64 (the workspace does not depend on the causal flag).
 static bool attn_bwd_tile_eligible(int N, int M, int D, int L, int R, int dtype, int causal) {
+    (void)causal;
     if (dtype == HSA_F32) return attn_bwd_tile_f32_eligible(N, M, D, L, R);
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
-    return nbw <= 2 || (nbw <= 4 && (causal != 0 || D <= 64));
-}
-// the tile passes run only with the causal mask at this radius and head size (16-bit types)
-static bool attn_bwd_tile_needs_causal(int R, int D, int dtype) {
-    return dtype != HSA_F32 && (R + TILE_Q - 1) / TILE_Q > 2 && D > 64;
+    return nbw <= 4;
 }
 
 static size_t bwd_gather_ws_floats(int B, int N, int H, int L, int R) {
@@ -718,7 +713,9 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
     p.scale_log2e = 1.4426950408889634f * p.scale;
     const int nbw = (R + TILE_Q - 1) / TILE_Q;
     const int NB = N / TILE_Q;
-    const int sb = NB % BWD_STRIP == 0 ? BWD_STRIP : 1;
+    // seven or nine leaf blocks per query block at 128 channels: one block per wavefront
+    const bool wide128 = nbw > 2 && !causal && D > 64;
+    const int sb = (NB % BWD_STRIP == 0 && !wide128) ? BWD_STRIP : 1;
     // The query pass finishes levels 1..4 (1..5 when it walks strips); the rows above them, the
     // root row and the rows past 2N-1 are summed from its partial rows by the trailing workgroups
     // of the key pass, one thread per four channels.
@@ -830,10 +827,7 @@ int hsa_build_parents_strided_bwd(const void *dout, const void *qp, const void *
 size_t hsa_attn_bwd_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype, int algo) {
     const bool tile = algo != HSA_ATTN_GATHER && hsa::attn_bwd_tile_eligible(N, M, D, L, R, dtype, -1);
     const size_t tile_fl = hsa::bwd_tile_ws_floats(B, N, H, D, L), gather_fl = hsa::bwd_gather_ws_floats(B, N, H, L, R);
-    size_t fl = tile ? tile_fl : gather_fl;
-    // the query does not say whether the call will be causal: where that decides between the two
-    // formulations, the automatic choice needs room for either
-    if (tile && algo == HSA_ATTN_AUTO && hsa::attn_bwd_tile_needs_causal(R, D, dtype) && gather_fl > fl) fl = gather_fl;
+    const size_t fl = tile ? tile_fl : gather_fl;
     return fl * sizeof(float);
 }
 
