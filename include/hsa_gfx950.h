@@ -324,6 +324,13 @@ size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int
 int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *out, const float *lse,
                        const void *dout, void *dq, void *dk, void *dv, void *workspace, size_t workspace_bytes,
                        int B, int N, int M, int H, int D, int L, int R, int causal, int dtype, void *stream);
+/*
+ * Query blocks one wavefront of hsa_attn_bwd_saved walks (no counterpart in the reference; for
+ * experiments and tests, results do not depend on it beyond rounding): 0 = automatic (eight where
+ * that many wavefronts still fill the chip, 64 channels per head and the sequence has a multiple
+ * of eight blocks; else four), 4, or 8 (used where the sequence allows it).  Process-wide.
+ */
+int hsa_attn_bwd_saved_tune(int strip_blocks);
 
 /*
  * hsa_attn_bwd for callers that cannot allocate device memory or hand over a workspace (code

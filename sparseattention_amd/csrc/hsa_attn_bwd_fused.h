@@ -2,8 +2,8 @@
 // window radius up to 16), for callers that kept the forward's output and log-sum-exp.
 //
 // The two-pass split (hsa_attn_bwd_tile.h) reads Q, dO and the leaf K / V twice: once per query
-// block for dQ, once per key block for dK / dV.  Here the wavefront that walks a strip of four
-// query blocks also finishes dK / dV of the strip's own four leaf key blocks: while a query block's
+// block for dQ, once per key block for dK / dV.  Here the wavefront that walks a strip of four or
+// eight query blocks also finishes dK / dV of the strip's own leaf key blocks: while a query block's
 // operands are in registers, its contribution to each leaf key block it attends is evaluated in
 // the second orientation (S[query, key], the queries in the MFMA contraction) and added to that
 // key block's accumulators; a key block is complete once the query block after it has been done.
@@ -11,33 +11,42 @@
 // the strip, and without the causal mask the one before it) is rebuilt from three pieces of saved
 // state instead of being exchanged: the neighbour's Q and dO rows, the forward's log-sum-exp of
 // those queries (P = exp2(logit - lse)) and delta = <dO, O> from the forward's output rows.
-// So every row of Q, dO, K, V is fetched once per strip plus one halo block in four (or two),
-// nothing leaves as a partial result except the rows of levels >= 6 (one fp32 row per strip and
-// level, summed by a small second launch), and there are no atomics.
+// So every row of Q, dO, K, V is fetched once per strip plus one halo block per strip (or two),
+// nothing leaves as a partial result except the rows of levels >= 6 (one fp32 row per 64 queries
+// and level, summed by a small second launch), and there are no atomics.
 //
 // What it costs: a wavefront carries the waiting key blocks' accumulators on top of everything the
-// query pass holds: about 350 registers at 64 channels per head, i.e. one wavefront per SIMD
-// (two at 32 channels).  With two per SIMD it spilled (85 registers; 32 with the accumulators
-// resting in LDS between iterations) and took 65 us at B8 H8 N2048 D64 against 56 us for the two
-// passes; with one per SIMD, nothing spilled and the next block's rows requested one block ahead it
-// takes 56.0 us against 56.6 us (same run, inputs rotated through 1 GiB), 29.7 against 34.6 us at
-// B16 H8 N512, 104 against 113 us at B8 H8 N4096; without the causal mask and at 32 channels the
-// two passes stay 3-4 % ahead.
+// query pass holds: 300-360 registers at 64 channels per head, i.e. one wavefront per SIMD (two at
+// 32 channels).  A block's rows therefore do not wait in registers: they are transferred from
+// global memory straight into the wavefront's LDS staging area one block ahead (hsa_lds_dma.h) and
+// read from there in operand form.  Measured at B8 H8 N2048 D64 with the causal mask, inputs
+// rotated through 1 GiB, both launches: 50.8 us against 56.4 us for the two passes (strips of
+// four blocks with the rows staged in registers: 56.0); with every load or every store removed
+// the same instruction stream takes 44 / 47 us, with both removed 36: the wavefront's own
+// instruction time is what is left to hide behind the memory system.
+// Strips of eight blocks where that still fills every wavefront slot: one neighbour's block per
+// 128 queries instead of per 64 (the far tree block and its partial rows change in the middle of
+// the strip, the leaf key blocks' accumulators just carry on).
 #pragma once
 
 #include "hsa_attn_bwd_tile.h"
+#include "hsa_lds_dma.h"
 
 namespace hsa {
+
+// blocks per strip forced through hsa_attn_bwd_saved_tune (0: automatic); defined in hsa_backward.hip
+int &bwd_fused_strip_knob();
 
 // Wavefronts per SIMD the fused pass is compiled for.
 constexpr int bwd_fused_waves(int D, bool causal) { return D <= 32 ? 2 : 1; }
 
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, int SB>
 __global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D, CAUSAL))))
 attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     using BT = BwdTile<T, D>;
     using M_ = Mma<T>;
-    constexpr int NBW = 1, SB = BWD_STRIP;
+    static_assert(SB == 4 || SB == 8, "a strip is one or two runs of four blocks (the 64 leaves under a level-6 node)");
+    constexpr int NBW = 1, FAR = BWD_STRIP;  // FAR: blocks that share the far tree block
     constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD, CPR = BT::CPR;
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
     constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
@@ -46,6 +55,12 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
     __shared__ __align__(16) float carry_mem[BWD_WPB * 2 * D];
     __shared__ __align__(16) float delta_mem[BWD_WPB * TILE_Q];
+    // A block's rows (Q, dO, entering leaf K / V, near tree K / V: six 16-row blocks) go from
+    // global memory straight into one of two staging areas per wavefront, unpadded, with the
+    // pieces of each row permuted (hsa_lds_dma.h); the neighbour's query block uses the area that
+    // is free at that moment.
+    constexpr int RB = 2 * D, ARR = TILE_Q * RB, STG = 6 * ARR, RPB = 256 / RB;
+    __shared__ __align__(16) unsigned char stage_mem[BWD_WPB * 2 * STG];
     // dK^T / dV^T of the key blocks that wait for the next query block: one when causal, two otherwise
     constexpr int NPARK = CAUSAL ? 1 : 2;
 
@@ -68,25 +83,31 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         for (int j = 0; j < NJ; ++j) { tk[j] = PK[slot][j]; tv[j] = PV[slot][j]; }
     };
 
-
     const int N = p.N, L = p.L, R = p.R, H = p.H;
     const int NB = N / TILE_Q, NS = NB / SB;
     const int h = unit % H;
     const int strip = (unit / H) % NS;
     const int b = unit / (H * NS);
     const int blk0 = strip * SB;
-    const int qs = blk0 * TILE_Q;  // first query of the strip
     const size_t rs = (size_t)H * D;
-    const uint16_t *Qb = p.q + ((size_t)b * N * H + h) * D + 8 * lchk;
-    const uint16_t *Gb = p.dout + ((size_t)b * N * H + h) * D + 8 * lchk;
-    const uint16_t *Ob = fp.out + ((size_t)b * N * H + h) * D + 8 * lchk;
-    const uint16_t *Kb = p.k + ((size_t)b * p.M * H + h) * D + 8 * lchk;
-    const uint16_t *Vb = p.v + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    const uint16_t *Q0 = p.q + ((size_t)b * N * H + h) * D, *G0 = p.dout + ((size_t)b * N * H + h) * D;
+    const uint16_t *O0 = fp.out + ((size_t)b * N * H + h) * D;
+    const uint16_t *K0 = p.k + ((size_t)b * p.M * H + h) * D, *V0 = p.v + ((size_t)b * p.M * H + h) * D;
+    const uint16_t *Kb = K0 + 8 * lchk, *Vb = V0 + 8 * lchk;
     uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
     uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    // staging: the piece of its row a lane fetches (in elements), the lane's operand addresses for
+    // the two contraction steps, and its own 16 bytes of a transfer
+    const uint32_t stg_base = lds_address(stage_mem) + wave * 2 * STG;
+    int pc8[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) pc8[i] = 8 * (lchk ^ (((i * RPI + lrow) / RPB) % CPR));
+    const uint32_t opa0 = stg_base + r16 * RB + ((g ^ ((r16 / RPB) % CPR)) << 4);
+    const uint32_t opa1 = stg_base + r16 * RB + ((((4 + g) % CPR) ^ ((r16 / RPB) % CPR)) << 4);
+    const uint32_t lin = stg_base + 16 * bt.lane;
 
     // ---- tree slot constants (same slot layout as the forward kernel) -------------------------
-    int t_lvl[NLD], t_add[NLD], t_xor[NLD], u_row[NLD];
+    int t_lvl[NLD], t_add[NLD], t_xor[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) {
         const int sl = i * RPI + lrow;
@@ -94,8 +115,6 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         else if (sl < 12) { t_lvl[i] = 2; t_add[i] = sl - 8; t_xor[i] = 0; }
         else if (sl < 14) { t_lvl[i] = 3; t_add[i] = sl - 12; t_xor[i] = 0; }
         else { t_lvl[i] = 4 + (sl - 14); t_add[i] = 0; t_xor[i] = 1; }
-        const int ul = 6 + sl;
-        u_row[i] = ul < L ? level_offset(N, ul) + ((qs >> ul) ^ 1) : -1;
     }
     auto near_row = [&](int i, int q0) {
         return t_lvl[i] < L ? level_offset(N, t_lvl[i]) + (((q0 >> t_lvl[i]) + t_add[i]) ^ t_xor[i]) : -1;
@@ -107,14 +126,27 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         pl = -1;
         return 4 + (sl - 14);
     };
+    // the far tree block (levels >= 6) of the run of four blocks that starts at query qr: one row
+    // per level, the same for the 64 queries of the run
     float b1U[4], b2U[4];
+    auto far_biases = [&](int qr) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ul1 = 6 + 4 * g + i;
-        b1U[i] = (ul1 < L && (!CAUSAL || ((qs >> ul1) & 1))) ? 0.f : NEG_INF;
-        const int ul2 = 6 + r16;
-        b2U[i] = (ul2 < L && (!CAUSAL || ((qs >> ul2) & 1))) ? 0.f : NEG_INF;
-    }
+        for (int i = 0; i < 4; ++i) {
+            const int ul1 = 6 + 4 * g + i;
+            b1U[i] = (ul1 < L && (!CAUSAL || ((qr >> ul1) & 1))) ? 0.f : NEG_INF;
+            const int ul2 = 6 + r16;
+            b2U[i] = (ul2 < L && (!CAUSAL || ((qr >> ul2) & 1))) ? 0.f : NEG_INF;
+        }
+    };
+    auto load_far = [&](int qr, u32x4_t (&rKu)[NLD], u32x4_t (&rVu)[NLD]) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int ul = 6 + i * RPI + lrow;
+            const int ur = ul < L ? level_offset(N, ul) + ((qr >> ul) ^ 1) : qr;
+            rKu[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)ur * rs);
+            rVu[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)ur * rs);
+        }
+    };
 
     // ---- loads ------------------------------------------------------------------------------
     auto load_block = [&](const uint16_t *base, int row0, u32x4_t (&dst)[NLD]) {
@@ -126,36 +158,47 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         kb = kb < 0 ? 0 : (kb >= NB ? NB - 1 : kb);
         return kb * TILE_Q;
     };
-    struct Stage {
-        u32x4_t q[NLD], g[NLD], k[NLD], v[NLD], kt[NLD], vt[NLD];
+    // transfers into the staging area at byte offset `area`
+    auto dma_block = [&](const uint16_t *base0, int row0, uint32_t dst) {
+        const uint16_t *ptr = base0 + (size_t)(row0 + lrow) * rs;
+        if constexpr (NLD == 2) lds_dma16_pair(ptr + pc8[0], ptr + (size_t)RPI * rs + pc8[1], dst, dst + 1024);
+        else lds_dma16(ptr + pc8[0], dst);
     };
-    auto request = [&](Stage &sg, int blk) {
+    auto request_dma = [&](int area, int blk) {  // 6 * NLD transfers
+        const uint32_t dst = stg_base + area;
         const int q0 = blk * TILE_Q;
-        load_block(Qb, q0, sg.q);
-        load_block(Gb, q0, sg.g);
+        dma_block(Q0, q0, dst);
+        dma_block(G0, q0, dst + ARR);
         const int row0 = leaf_row0(blk - NBW + NKL - 1);
-        load_block(Kb, row0, sg.k);
-        load_block(Vb, row0, sg.v);
+        dma_block(K0, row0, dst + 2 * ARR);
+        dma_block(V0, row0, dst + 3 * ARR);
+        const uint16_t *kp[NLD], *vp[NLD];
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int tr = near_row(i, q0);
-            sg.kt[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(tr < 0 ? q0 : tr) * rs);
-            sg.vt[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(tr < 0 ? q0 : tr) * rs);
+            kp[i] = K0 + (size_t)(tr < 0 ? q0 : tr) * rs + pc8[i];
+            vp[i] = V0 + (size_t)(tr < 0 ? q0 : tr) * rs + pc8[i];
+        }
+        if constexpr (NLD == 2) {
+            lds_dma16_pair(kp[0], kp[1], dst + 4 * ARR, dst + 4 * ARR + 1024);
+            lds_dma16_pair(vp[0], vp[1], dst + 5 * ARR, dst + 5 * ARR + 1024);
+        } else {
+            lds_dma16(kp[0], dst + 4 * ARR);
+            lds_dma16(vp[0], dst + 5 * ARR);
         }
     };
-    // a neighbouring strip's query block: rows of Q, dO and of the forward's output, and the
-    // forward's log-sum-exp of its queries (4g + i)
-    struct Halo {
-        u32x4_t q[NLD], g[NLD], o[NLD];
-        float lse4[4];
-    };
-    auto request_halo = [&](Halo &hl, int qb) {
+    // a neighbouring strip's query block: 3 * NLD transfers (Q, dO, forward output); the
+    // log-sum-exp values of its queries (4g + i) go to registers and are requested first, so that
+    // the wait that follows the transfers covers them
+    auto request_halo_dma = [&](int area, int qb, float (&lse4)[4]) {
         qb = qb < 0 ? 0 : (qb >= NB ? NB - 1 : qb);
-        load_block(Qb, qb * TILE_Q, hl.q);
-        load_block(Gb, qb * TILE_Q, hl.g);
-        load_block(Ob, qb * TILE_Q, hl.o);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) hl.lse4[i] = fp.lse[((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h];
+        for (int i = 0; i < 4; ++i) lse4[i] = fp.lse[((size_t)b * N + qb * TILE_Q + 4 * g + i) * H + h];
+        asm volatile("" ::: "memory");
+        const uint32_t dst = stg_base + area;
+        dma_block(Q0, qb * TILE_Q, dst);
+        dma_block(G0, qb * TILE_Q, dst + ARR);
+        dma_block(O0, qb * TILE_Q, dst + 2 * ARR);
     };
 
     // contribution of one query block (operands Qf/Gf, their transposes, the queries' lse and
@@ -190,36 +233,42 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             tv[j] = M_::k16(GT[j], pk, tv[j]);
         }
     };
-    // contribution of a neighbouring strip's query block to one of this strip's key blocks
-    auto halo_contrib = [&](const Halo &hl, int qb, const u32x4_t (&Kf)[KS], const u32x4_t (&Vf)[KS], int kb,
-                            f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
-        // delta[q] = <dO[q], O[q]>: the lanes that share a row sum their pieces
+    // contribution of a neighbouring strip's staged query block (area offset as a compile-time
+    // tag) to one of this strip's key blocks
+    auto halo_contrib = [&](auto area_tag, const float (&lse4)[4], int qb, const u32x4_t (&Kf)[KS],
+                            const u32x4_t (&Vf)[KS], int kb, f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
+        constexpr int OFF = decltype(area_tag)::value;
+        u32x4_t Qf[KS], Gf[KS], gw[NLD], ow[NLD];
+        if constexpr (KS == 2) {
+            lds_read16_x4<OFF, OFF, OFF + ARR, OFF + ARR>(opa0, opa1, opa0, opa1, Qf[0], Qf[1], Gf[0], Gf[1]);
+            lds_read16_x4<OFF + ARR, OFF + ARR + 1024, OFF + 2 * ARR, OFF + 2 * ARR + 1024>(lin, lin, lin, lin, gw[0],
+                                                                                          gw[1], ow[0], ow[1]);
+        } else {
+            lds_read16_x4<OFF, OFF + ARR, OFF + ARR, OFF + 2 * ARR>(opa0, opa0, lin, lin, Qf[0], Gf[0], gw[0], ow[0]);
+        }
+        // delta[q] = <dO[q], O[q]>: the lanes that share a row sum their pieces (both rows carry
+        // the same permutation of pieces)
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             float s = 0.f;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const uint32_t gw = hl.g[i][w], ow = hl.o[i][w];
-                s = fmaf(to_float<T>((uint16_t)(gw & 0xffffu)), to_float<T>((uint16_t)(ow & 0xffffu)), s);
-                s = fmaf(to_float<T>((uint16_t)(gw >> 16)), to_float<T>((uint16_t)(ow >> 16)), s);
+                const uint32_t a = gw[i][w], o = ow[i][w];
+                s = fmaf(to_float<T>((uint16_t)(a & 0xffffu)), to_float<T>((uint16_t)(o & 0xffffu)), s);
+                s = fmaf(to_float<T>((uint16_t)(a >> 16)), to_float<T>((uint16_t)(o >> 16)), s);
             }
 #pragma unroll
             for (int m = 1; m < CPR; m <<= 1) s += __shfl_xor(s, m, 64);
             if (lchk == 0) delta_lds[i * RPI + lrow] = s;
         }
-        u32x4_t Qf[KS], Gf[KS];
         u32x2_t QT[NJ], GT[NJ];
-        bt.put(0, hl.q);
-        bt.put(1, hl.g);
-        bt.get(0, Qf);
-        bt.get(1, Gf);
         bt.transpose(Qf, QT);
         bt.transpose(Gf, GT);
         float del4[4];
         const f32x4 dl = *reinterpret_cast<const f32x4 *>(delta_lds + 4 * g);
 #pragma unroll
         for (int i = 0; i < 4; ++i) del4[i] = dl[i];
-        leaf_contrib(Qf, Gf, QT, GT, hl.lse4, del4, Kf, Vf, qb, kb, tk, tv);
+        leaf_contrib(Qf, Gf, QT, GT, lse4, del4, Kf, Vf, qb, kb, tk, tv);
     };
     auto store_key_block = [&](int kb, const f32x4 (&tk)[NJ], const f32x4 (&tv)[NJ]) {
         bt.put_result(0, tk, 1.0f);
@@ -235,28 +284,21 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 
     // everything the first block needs is requested before anything is consumed
     u32x4_t Kc[NKB][KS], Vc[NKB][KS];
-    Stage sgs[2];
-    Stage &sg = sgs[0];
-    Halo halo;
+    u32x4_t rKu[NLD], rVu[NLD];  // the far block's rows on their way
+    float halo_lse4[4];
+    using Area0 = std::integral_constant<int, 0>;
+    using Area1 = std::integral_constant<int, STG>;
     const bool left_halo = !CAUSAL && blk0 > 0, right_halo = blk0 + SB < NB;  // uniform
     {
-        u32x4_t rKu[NLD], rVu[NLD], rKh[NKL][NLD], rVh[NKL][NLD];
-#pragma unroll
-        for (int i = 0; i < NLD; ++i) {
-            rKu[i] = *reinterpret_cast<const u32x4_t *>(Kb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
-            rVu[i] = *reinterpret_cast<const u32x4_t *>(Vb + (size_t)(u_row[i] < 0 ? qs : u_row[i]) * rs);
-        }
+        u32x4_t rKh[NKL][NLD], rVh[NKL][NLD];
+        load_far(blk0 * TILE_Q, rKu, rVu);
 #pragma unroll
         for (int c = 0; c + 1 < NKL; ++c) {
             load_block(Kb, leaf_row0(blk0 - NBW + c), rKh[c]);
             load_block(Vb, leaf_row0(blk0 - NBW + c), rVh[c]);
         }
-        if constexpr (!CAUSAL) request_halo(halo, blk0 - 1);
-        request(sg, blk0);
-        bt.put(2, rKu);
-        bt.put(3, rVu);
-        bt.get(2, Kc[NKL + 1]);
-        bt.get(3, Vc[NKL + 1]);
+        if constexpr (!CAUSAL) request_halo_dma(STG, blk0 - 1, halo_lse4);
+        request_dma(0, blk0);
 #pragma unroll
         for (int c = 0; c + 1 < NKL; ++c) {
             bt.put(2, rKh[c]);
@@ -271,33 +313,52 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         f32x4 tk[NJ], tv[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-        if (left_halo) halo_contrib(halo, blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
+        wait_vmem_all_but<6 * NLD>();  // everything older than the first block's transfers
+        if (left_halo) halo_contrib(Area1{}, halo_lse4, blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
         park_put(0, tk, tv);
     }
-    // partial rows of the far block, summed over the strip
+    // partial rows of the far block, summed over a run of four blocks
     f32x4 fk[NJ], fv[NJ];
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 
-#pragma unroll
-    for (int it = 0; it < SB; ++it) {
+    // one query block; PAR = parity of `it`, the block's index within the strip
+    auto body = [&](auto par_tag, const int it) {
+        constexpr int PAR = decltype(par_tag)::value;
         const int blk = blk0 + it;
         const int q0 = blk * TILE_Q;
-        Stage &sg = sgs[it & 1];
-        if (it + 1 < SB) request(sgs[(it + 1) & 1], blk + 1);  // the next block's rows, one block ahead
+        if ((it & (FAR - 1)) == 0) {
+            // a new run: its far block (requested a block ahead), nothing summed yet
+            bt.put(2, rKu);
+            bt.put(3, rVu);
+            bt.get(2, Kc[NKL + 1]);
+            bt.get(3, Vc[NKL + 1]);
+            far_biases(q0);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+        }
         u32x4_t Qf[KS], Gf[KS];
-        bt.put(0, sg.q);
-        bt.put(1, sg.g);
-        bt.put(2, sg.k);
-        bt.put(3, sg.v);
-        bt.get(0, Qf);
-        bt.get(1, Gf);
-        bt.get(2, Kc[NKL - 1]);
-        bt.get(3, Vc[NKL - 1]);
-        bt.put(2, sg.kt);
-        bt.put(3, sg.vt);
-        bt.get(2, Kc[NKL]);
-        bt.get(3, Vc[NKL]);
+        // the next block's rows (after the last block: the neighbour's query block) into the other
+        // area, whose reads finished an iteration ago; then everything older is here
+        // The counter the waits look at retires loads, transfers and stores in the order of issue,
+        // so the wait names how many younger operations may still be in flight: the transfers
+        // just requested plus the previous block's stores, which follow this block's request in
+        // program order.  Only stores that are certainly issued are counted (dQ: NLD; the finished
+        // leaf key block: 2 NLD from the strip's second block on; near tree rows: 2 NLD, some
+        // lane always has a row); counting too few only waits longer.
+        if (it + 1 < SB) {
+            request_dma((PAR ^ 1) * STG, blk + 1);
+            if (it == 0) wait_vmem_all_but<6 * NLD>();
+            else if (it == 1) wait_vmem_all_but<6 * NLD + 3 * NLD>();
+            else wait_vmem_all_but<6 * NLD + 5 * NLD>();
+        } else {
+            request_halo_dma((PAR ^ 1) * STG, blk0 + SB, halo_lse4);
+            wait_vmem_all_but<3 * NLD + 4 + 5 * NLD>();  // SB >= 4: the block before stored all of the above
+        }
+        if constexpr (KS == 2)
+            lds_read16_6x2<PAR * STG, ARR>(opa0, opa1, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
+        else
+            lds_read16_6x1<PAR * STG, ARR>(opa0, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
+        if constexpr (SB > FAR)
+            if ((it & (FAR - 1)) == FAR - 1 && it + 1 < SB) load_far(q0 + TILE_Q, rKu, rVu);  // the next run's far block
 
         int t_row[NLD];
 #pragma unroll
@@ -415,12 +476,12 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             lse4[i] = __shfl(lse, 4 * g + i, 64);
             del4[i] = __shfl(delta, 4 * g + i, 64);
         }
-        if (it == SB - 1) request_halo(halo, blk0 + SB);  // arrives while the rest of the last block is computed
         // the strip's own leaf key blocks this query block reaches, oldest first: the block before
-        // the query block is complete afterwards and leaves; the others rest in LDS
+        // the query block is complete afterwards and leaves; the others wait in registers
 #pragma unroll
         for (int c = 0; c < NKL; ++c) {
-            const int j = it - NBW + c;  // key block within the strip
+            const int j = it - NBW + c;                                // key block within the strip
+            const int SLOT = ((PAR + NBW + c) & 1) & (NPARK - 1);      // j % NPARK (NBW + it + c has j's parity)
             if (j >= 0 && j < SB) {
                 f32x4 tk[NJ], tv[NJ];
                 const bool fresh = c == NKL - 1 && (CAUSAL || j > 0);  // nobody has contributed yet
@@ -428,11 +489,11 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 #pragma unroll
                     for (int jj = 0; jj < NJ; ++jj) { tk[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; }
                 } else {
-                    park_get(j % NPARK, tk, tv);
+                    park_get(SLOT, tk, tv);
                 }
                 leaf_contrib(Qf, Gf, QT, GT, lse4, del4, Kc[c], Vc[c], blk, blk0 + j, tk, tv);
                 if (c == 0) store_key_block(blk0 + j, tk, tv);
-                else park_put(j % NPARK, tk, tv);
+                else park_put(SLOT, tk, tv);
             }
         }
 #pragma unroll
@@ -467,7 +528,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) {
                         const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
-                        if (it & 1) {
+                        if constexpr (PAR == 1) {
                             const f32x4 ck = *reinterpret_cast<const f32x4 *>(carry + ch);
                             const f32x4 cv = *reinterpret_cast<const f32x4 *>(carry + D + ch);
                             tk[j] += ck;
@@ -478,7 +539,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
                         }
                     }
                 }
-                const bool five_final = (it & 1) != 0;
+                constexpr bool five_final = PAR == 1;
                 bt.put_result(0, tk, 1.0f);
                 bt.put_result(1, tv, 1.0f);
 #pragma unroll
@@ -498,39 +559,56 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             }
         }
 
+        // levels >= 6: the partial rows of the run of four blocks that ends here
+        if ((it & (FAR - 1)) == FAR - 1) {
+            const int lvl = 6 + r16;
+            const int LF = L - 6;
+            if (lvl < L) {
+                const int NR = NB / FAR;
+                float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
+                const size_t po = ((((size_t)b * NR + blk / FAR) * H + h) * LF + (lvl - 6)) * D;
+                float *pkp = far + po;
+                float *pvp = far + (size_t)p.B * NR * H * LF * D + po;
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                    *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
+                    *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
+                }
+            }
+        }
+
         // slide the leaf window by one block
 #pragma unroll
         for (int c = 0; c + 1 < NKL; ++c) {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) { Kc[c][ks] = Kc[c + 1][ks]; Vc[c][ks] = Vc[c + 1][ks]; }
         }
+    };
+
+    if constexpr (SB == FAR) {
+#pragma unroll
+        for (int ip = 0; ip < SB / 2; ++ip) {
+            body(std::integral_constant<int, 0>{}, 2 * ip);
+            body(std::integral_constant<int, 1>{}, 2 * ip + 1);
+        }
+    } else {
+#pragma unroll 1  // unrolled it is slower (53.6 against 52.2 us at B8 H8 N2048 D64)
+        for (int ip = 0; ip < SB / 2; ++ip) {
+            body(std::integral_constant<int, 0>{}, 2 * ip);
+            body(std::integral_constant<int, 1>{}, 2 * ip + 1);
+        }
     }
 
     // the strip's last key block: the query block after the strip reaches it (the block sits in
     // the first operand slot after the last slide)
     {
+        static_assert(SB % 2 == 0, "the neighbour's block is staged in the first area");
         f32x4 tk[NJ], tv[NJ];
-        park_get((SB - 1) % NPARK, tk, tv);
-        if (right_halo) halo_contrib(halo, blk0 + SB, Kc[0], Vc[0], blk0 + SB - 1, tk, tv);
+        park_get(((SB - 1) & 1) & (NPARK - 1), tk, tv);
+        wait_vmem_all_but<0>();
+        if (right_halo) halo_contrib(Area0{}, halo_lse4, blk0 + SB, Kc[0], Vc[0], blk0 + SB - 1, tk, tv);
         store_key_block(blk0 + SB - 1, tk, tv);
-    }
-
-    // levels >= 6: the strip's partial rows
-    {
-        const int lvl = 6 + r16;
-        const int LF = L - 6;
-        if (lvl < L) {
-            float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
-            const size_t po = ((((size_t)b * NS + strip) * H + h) * LF + (lvl - 6)) * D;
-            float *pkp = far + po;
-            float *pvp = far + (size_t)p.B * NS * H * LF * D + po;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
-                const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
-                *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
-                *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
-            }
-        }
     }
 }
 
@@ -539,22 +617,34 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 template <typename T>
 __global__ void __launch_bounds__(BWD_WPB * 64) attn_bwd_reduce_kernel(BwdTileParams p, int D) {
     using S = typename T::storage;
-    bwd_reduce_rows<T>(p.partial, reinterpret_cast<S *>(p.dk), reinterpret_cast<S *>(p.dv), p.B, p.N, p.M, p.H, D, p.L,
-                       p.causal, p.red_first_row, p.red_lg_sb, (size_t)blockIdx.x * (BWD_WPB * 64) + threadIdx.x);
+    bwd_reduce_rows<T, BWD_FUSED_RED_SPLIT>(p.partial, reinterpret_cast<S *>(p.dk), reinterpret_cast<S *>(p.dv), p.B, p.N,
+                                            p.M, p.H, D, p.L, p.causal, p.red_first_row, p.red_lg_sb,
+                                            (size_t)blockIdx.x * (BWD_WPB * 64) + threadIdx.x);
 }
 
 template <typename T, int D>
 int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
 
+// strips of eight blocks where the sequence has that many (one neighbour's block per 128 queries
+// instead of per 64, every wavefront slot of the chip filled once at B8 H8 N2048), else of four
 #define HSA_BWD_FUSED_INSTANTIATE(T, D)                                                                     \
     template <>                                                                                             \
     int attn_bwd_fused_launch_td<T, D>(const BwdFusedParams &fp, bool causal, hipStream_t st) {             \
         BwdFusedParams q = fp;                                                                              \
-        q.t.n_units = fp.t.n_units / BWD_STRIP;                                                             \
+        const int NB = fp.t.N / TILE_Q;                                                                     \
+        const bool fills = (long)(fp.t.n_units / 8) >= 1024; /* one wavefront per SIMD on 256 CUs */       \
+        const int knob = bwd_fused_strip_knob();                                                            \
+        const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D == 64 && fills))) ? 8 : 4;             \
+        q.t.n_units = fp.t.n_units / sb;                                                                    \
         q.t.red_lg_sb = 2;                                                                                  \
         const int nwg = (q.t.n_units + BWD_WPB - 1) / BWD_WPB;                                              \
-        if (causal) attn_bwd_tile_fused_kernel<T, D, true><<<nwg, BWD_WPB * 64, 0, st>>>(q);                \
-        else attn_bwd_tile_fused_kernel<T, D, false><<<nwg, BWD_WPB * 64, 0, st>>>(q);                      \
+        if (sb == 8) {                                                                                      \
+            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 8><<<nwg, BWD_WPB * 64, 0, st>>>(q);         \
+            else attn_bwd_tile_fused_kernel<T, D, false, 8><<<nwg, BWD_WPB * 64, 0, st>>>(q);               \
+        } else {                                                                                            \
+            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 4><<<nwg, BWD_WPB * 64, 0, st>>>(q);         \
+            else attn_bwd_tile_fused_kernel<T, D, false, 4><<<nwg, BWD_WPB * 64, 0, st>>>(q);               \
+        }                                                                                                   \
         int rc = check_launch("attn_bwd_tile_fused_kernel");                                                \
         if (rc != HSA_OK || q.t.red_wgs == 0) return rc;                                                    \
         attn_bwd_reduce_kernel<T><<<q.t.red_wgs, BWD_WPB * 64, 0, st>>>(q.t, D);                            \

@@ -49,6 +49,8 @@ struct BwdFusedParams {
 };
 
 constexpr int BWD_WPB = 4;  // wavefronts per workgroup
+// threads that share one output row piece in the one-pass variant's second launch
+constexpr int BWD_FUSED_RED_SPLIT = 8;
 
 // Hardware hands consecutive workgroup ids to the 8 XCDs in turn; with this remap workgroups that
 // are consecutive in the returned index run on the same XCD, so neighbouring strips (which share
@@ -523,7 +525,7 @@ attn_bwd_tile_query_kernel(BwdTileParams p) {
     }
 }
 
-template <typename T>
+template <typename T, int SPLIT = 1>
 __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
                                                 typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D,
                                                 int L, int causal, int first_row, int lg_sb, size_t t);
@@ -704,14 +706,18 @@ attn_bwd_tile_key_kernel(BwdTileParams p) {
 // Rows from first_row on (a level the query pass left unfinished, up to anything above row 2N-2):
 // node (l, p) sums the partial rows of the query blocks (levels 4, 5) or strips (levels >= 6)
 // under its sibling; nodes nobody attends (the root, right-hand nodes when causal, rows past
-// 2N-1) get zeros.  One thread per (batch, row, head, four channels), index t.  lg_sb = log2 of
-// the blocks per strip of the query pass.
-template <typename T>
+// 2N-1) get zeros.  SPLIT consecutive threads per (batch, row, head, four channels) share the
+// partial rows of one output (the top levels have the most: one per strip of the sequence),
+// index t.  lg_sb = log2 of the blocks per strip of the query pass.
+template <typename T, int SPLIT>
 __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partial, typename T::storage *__restrict__ dk,
                                                 typename T::storage *__restrict__ dv, int B, int N, int M, int H, int D,
                                                 int L, int causal, int first_row, int lg_sb, size_t t) {
     using S = typename T::storage;
     struct alignas(4 * sizeof(S)) Pack { S e[4]; };
+    static_assert(SPLIT == 1 || SPLIT == 2 || SPLIT == 4 || SPLIT == 8, "lanes that share an output");
+    const int sub = (int)(t % SPLIT);
+    t /= SPLIT;
     const int D4 = D / 4;
     const size_t per_b = (size_t)(M - first_row) * H * D4;
     if (t >= (size_t)B * per_b) return;
@@ -746,6 +752,23 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
             }
             // eight independent 16-byte loads per tensor in flight per round trip
             int i = 0;
+            if constexpr (SPLIT > 1) {
+                for (i = sub; i + 3 * SPLIT < n; i += 4 * SPLIT) {
+                    f32x4 a[4], c[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        a[u] = *reinterpret_cast<const f32x4 *>(pk + (size_t)(i + u * SPLIT) * stride);
+                        c[u] = *reinterpret_cast<const f32x4 *>(pv + (size_t)(i + u * SPLIT) * stride);
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) { vk += a[u]; vv += c[u]; }
+                }
+                for (; i < n; i += SPLIT) {
+                    vk += *reinterpret_cast<const f32x4 *>(pk + (size_t)i * stride);
+                    vv += *reinterpret_cast<const f32x4 *>(pv + (size_t)i * stride);
+                }
+                i = n;
+            }
             for (; i + 8 <= n; i += 8) {
                 f32x4 a[8], c[8];
 #pragma unroll
@@ -761,6 +784,17 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
                 vv += *reinterpret_cast<const f32x4 *>(pv + (size_t)i * stride);
             }
         }
+    }
+    if constexpr (SPLIT > 1) {
+        // the lanes of a group are neighbours in the wavefront and all of them get here
+#pragma unroll
+        for (int m = 1; m < SPLIT; m <<= 1)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                vk[u] += __shfl_xor(vk[u], m, 64);
+                vv[u] += __shfl_xor(vv[u], m, 64);
+            }
+        if (sub != 0) return;
     }
     const size_t o = ((size_t)b * M + row) * H * D + (size_t)h * D + d;
     Pack ok, ov;

@@ -733,6 +733,10 @@ static int attn_bwd_tile_typed(const void *q, const void *k, const void *v, cons
 }
 
 // ---- one-pass backward on saved forward state (hsa_attn_bwd_fused.h) ---------------------------
+int &bwd_fused_strip_knob() {
+    static int v = 0;
+    return v;
+}
 template <typename T, int D>
 int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
 
@@ -771,7 +775,7 @@ static int attn_bwd_fused_typed(const void *q, const void *k, const void *v, con
     // summed from the strips' partial rows by a second, small launch
     int first = level_offset(N, 6);
     if (first > 2 * N - 2) first = 2 * N - 2;
-    const size_t red_threads = (size_t)B * (M - first) * H * (D / 4);
+    const size_t red_threads = (size_t)B * (M - first) * H * (D / 4) * BWD_FUSED_RED_SPLIT;
     const size_t red_wgs = (red_threads + BWD_WPB * 64 - 1) / (BWD_WPB * 64);
     if (red_wgs > 0x3fffffffUL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.causal = causal != 0;
@@ -875,6 +879,13 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
         case HSA_BF16: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
     }
     return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+int hsa_attn_bwd_saved_tune(int strip_blocks) {
+    if (strip_blocks != 0 && strip_blocks != 4 && strip_blocks != 8)
+        return hsa::fail(HSA_ERR_INVALID, "strip length %d (0, 4 or 8)", strip_blocks);
+    hsa::bwd_fused_strip_knob() = strip_blocks;
+    return HSA_OK;
 }
 
 size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype) {

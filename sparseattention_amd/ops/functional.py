@@ -383,12 +383,12 @@ class BuildParentNodesFunc(torch.autograd.Function):
 # Which backward `hierarchical_attention` uses.  Two formulations exist: two passes over Q, dO and
 # the leaf K / V (any shape the tile kernels take), and one pass that works from the forward's
 # output and one log-sum-exp per (query, head), which the forward then keeps (16-bit types, 32 / 64
-# channels per head, window radius up to 16).  The one pass moves less (0.86 of the two passes' HBM
-# traffic at B8 H8 N2048 D64) and is as fast or faster with the causal mask at 64 channels per head
-# (56.0 against 56.6 us there, 29.7 against 34.6 us at B16 H8 N512); without the mask and at 32
-# channels the two passes are 3-4 % ahead.
-#   None (default): the one pass where it measured at least as fast (causal, 64 channels per head)
-#   True / False:   the one pass wherever it applies / never
+# channels per head, window radius up to 16).  The one pass moves less (0.76 of the two passes' HBM
+# traffic at B8 H8 N2048 D64) and measured faster on every shape tried (50.8 against 56.4 us there,
+# 29.6 against 34.7 us at B16 H8 N512, 64.0 against 68.9 us at B2 H16 N8192 D32, 53.8 against 58.7 us
+# at B8 H8 N2048 without the causal mask).
+#   None (default): the one pass wherever it is built
+#   True / False:   the same / never
 # Process-wide; read when the forward runs.
 one_pass_backward = None
 
@@ -396,7 +396,7 @@ one_pass_backward = None
 def _use_one_pass(Q, K, window_size, causal) -> bool:
     if one_pass_backward is False or not saved_state_backward_available(Q, K, window_size):
         return False
-    return True if one_pass_backward else (bool(causal) and Q.shape[3] == 64)
+    return True
 
 
 class HierarchicalAttentionFunc(torch.autograd.Function):

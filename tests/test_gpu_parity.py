@@ -1073,7 +1073,7 @@ def test_attention_backward_wide_window_128_channels_both_formulations(dtype, ca
 
 
 SAVED_BWD_CASES = [(2, 64, 2, 64, 16), (1, 128, 3, 64, 5), (2, 256, 4, 32, 16), (1, 512, 2, 64, 0), (2, 1024, 8, 64, 16),
-                   (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1)]
+                   (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1), (1, 128, 1, 32, 16), (1, 4096, 3, 64, 13)]
 
 
 @pytest.mark.parametrize("case", SAVED_BWD_CASES)
@@ -1118,13 +1118,23 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
     assert (lse.double().cpu() - want_lse).abs().max() < 2e-2
     got = fn.attention_backward_saved(gd, qd, kd, vd, out, lse, R, causal)
     two = fn.attention_backward(gd, qd, kd, vd, R, causal)
+    # strips of four and of eight query blocks per wavefront (eight: one neighbour's block per 128
+    # queries, the far tree block changes in the middle of the strip)
+    for strip in (4, 8):
+        assert _lib.lib().hsa_attn_bwd_saved_tune(strip) == 0
+        try:
+            forced = fn.attention_backward_saved(gd, qd, kd, vd, out, lse, R, causal)
+        finally:
+            _lib.lib().hsa_attn_bwd_saved_tune(0)
+        for name, g1, ref in zip(("dQ", "dK", "dV"), forced, (qr.grad, kr.grad, vr.grad)):
+            _grad_close(g1, ref, dtype, "%s one pass, strips of %d, causal=%s" % (name, strip, causal))
     for name, g1, g2, ref in zip(("dQ", "dK", "dV"), got, two, (qr.grad, kr.grad, vr.grad)):
         _grad_close(g1, ref, dtype, "%s one pass, causal=%s" % (name, causal))
         scale = max(1.0, float(ref.abs().max()))
         assert (g1.float() - g2.float()).abs().max() <= 2e-2 * scale, "%s: one pass vs two passes" % name
-    # and through the autograd function: the switch forces either formulation, the default picks
-    # the one pass with the causal mask at 64 channels per head
-    for flag, ref in ((False, two), (True, got), (None, got if (causal and D == 64) else two)):
+    # and through the autograd function: the switch forces either formulation, the default is the
+    # one pass wherever it is built
+    for flag, ref in ((False, two), (True, got), (None, got)):
         qa, ka, va = (x.clone().requires_grad_(True) for x in (qd, kd, vd))
         fn.one_pass_backward = flag
         try:
