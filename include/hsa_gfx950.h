@@ -333,6 +333,23 @@ int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *
 int hsa_attn_bwd_saved_tune(int strip_blocks);
 
 /*
+ * Backward of the span attention from caller-supplied tables, replacing
+ * HierarchicalAttentionFunc.backward for tables that are not the canonical ones
+ * (hierarchical_attention/ops/functional.py:171-264): like the reference's kernels
+ * (ops/triton/sparse_attn.py:185-623) it takes each query's key rows and dead slots from
+ * idx [N, L] / mask [N, L] (mask NULL: nothing masked; an entry outside [0, M) is a dead slot),
+ * keeps the tree's row layout (level l starts at row 2N - (N >> (l-1)), a node of level l collects
+ * from 2^l consecutive queries) and reads from gather [rows, 3] only each node row's first
+ * attending query (column 0; -1: none).  `causal` restricts the window to keys <= the query, as the
+ * reference does when a mask table is given.  Per-query / per-key-row gather kernels, any head
+ * size, fp32 workspaces of hsa_attn_bwd_workspace_bytes(..., HSA_ATTN_GATHER) bytes; deterministic.
+ */
+int hsa_attn_bwd_tables(const void *q, const void *k, const void *v, const void *dout, const int32_t *idx,
+                        const uint8_t *mask, const int32_t *gather, void *dq, void *dk, void *dv, void *workspace,
+                        size_t workspace_bytes, int B, int N, int M, int H, int D, int L, int R, int causal, int dtype,
+                        void *stream);
+
+/*
  * hsa_attn_bwd for callers that cannot allocate device memory or hand over a workspace (code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference: its backward allocates its workspaces through torch

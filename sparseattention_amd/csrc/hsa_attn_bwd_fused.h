@@ -332,8 +332,12 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             bt.get(2, Kc[NKL + 1]);
             bt.get(3, Vc[NKL + 1]);
             far_biases(q0);
+            // the strip's second run goes on summing the levels above 6, whose nodes it shares
+            // with the first; level 6 (the lanes of slot 0) starts over
+            if (it == 0 || r16 == 0) {
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+                for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+            }
         }
         u32x4_t Qf[KS], Gf[KS];
         // the next block's rows (after the last block: the neighbour's query block) into the other
@@ -559,14 +563,16 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             }
         }
 
-        // levels >= 6: the partial rows of the run of four blocks that ends here
+        // levels >= 6: partial rows, laid out per run of four blocks.  Level 6: the run that ends
+        // here; the levels above: the strip, stored with its last block in the strip's first run
         if ((it & (FAR - 1)) == FAR - 1) {
             const int lvl = 6 + r16;
             const int LF = L - 6;
-            if (lvl < L) {
+            if (lvl < L && (it == SB - 1 || r16 == 0)) {
                 const int NR = NB / FAR;
                 float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
-                const size_t po = ((((size_t)b * NR + blk / FAR) * H + h) * LF + (lvl - 6)) * D;
+                const int run = r16 == 0 ? blk / FAR : blk0 / FAR;
+                const size_t po = ((((size_t)b * NR + run) * H + h) * LF + (lvl - 6)) * D;
                 float *pkp = far + po;
                 float *pvp = far + (size_t)p.B * NR * H * LF * D + po;
 #pragma unroll
@@ -636,7 +642,7 @@ int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t 
         const int knob = bwd_fused_strip_knob();                                                            \
         const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D == 64 && fills))) ? 8 : 4;             \
         q.t.n_units = fp.t.n_units / sb;                                                                    \
-        q.t.red_lg_sb = 2;                                                                                  \
+        q.t.red_lg_sb = sb == 8 ? 3 : 2;                                                                    \
         const int nwg = (q.t.n_units + BWD_WPB - 1) / BWD_WPB;                                              \
         if (sb == 8) {                                                                                      \
             if (causal) attn_bwd_tile_fused_kernel<T, D, true, 8><<<nwg, BWD_WPB * 64, 0, st>>>(q);         \

@@ -732,7 +732,7 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
         while (row >= level_offset(N, lvl + 1)) ++lvl;
         const int pidx = row - level_offset(N, lvl);
         if (!causal || (pidx & 1) == 0) {
-            const int NB = N / TILE_Q, NS = NB >> lg_sb;
+            const int NB = N / TILE_Q;
             const int blk0 = (pidx ^ 1) << (lvl - 4);  // first query block under the sibling
             const float *pk, *pv;
             size_t stride;
@@ -743,12 +743,18 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
                 pk = partial + (((size_t)b * NB + blk0) * H + h) * 2 * D + (size_t)(lvl - 4) * D + d;
                 pv = pk + (size_t)B * NB * H * 2 * D;
             } else {
+                // lg_sb == 3 (the one-pass variant's strips of eight blocks): the area is laid out per
+                // run of four blocks; level 6 has a row per run, the levels above one per strip, in
+                // the strip's first run
                 const int LF = L - 6;
-                n = (1 << (lvl - 4)) >> lg_sb;
-                stride = (size_t)H * LF * D;
+                const int lgl = lg_sb == 3 ? 2 : lg_sb;             // layout granularity
+                const int lg = (lg_sb == 3 && lvl == 6) ? 2 : lg_sb;  // blocks summed into one row
+                const int NR = NB >> lgl;
+                n = (1 << (lvl - 4)) >> lg;
+                stride = ((size_t)H * LF * D) << (lg - lgl);
                 const float *far = partial + 2 * (size_t)B * NB * H * 2 * D;
-                pk = far + (((size_t)b * NS + (blk0 >> lg_sb)) * H + h) * LF * D + (size_t)(lvl - 6) * D + d;
-                pv = pk + (size_t)B * NS * H * LF * D;
+                pk = far + (((size_t)b * NR + (blk0 >> lgl)) * H + h) * LF * D + (size_t)(lvl - 6) * D + d;
+                pv = pk + (size_t)B * NR * H * LF * D;
             }
             // eight independent 16-byte loads per tensor in flight per round trip
             int i = 0;

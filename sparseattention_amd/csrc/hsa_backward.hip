@@ -204,7 +204,8 @@ __global__ void __launch_bounds__(256)
 attn_bwd_query_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ K,
                       const typename T::storage *__restrict__ V, const typename T::storage *__restrict__ dO,
                       typename T::storage *__restrict__ dQ, float *__restrict__ Pw, float *__restrict__ DS, int B,
-                      int N, int M, int H, int D, int L, int R, int causal, float scale) {
+                      int N, int M, int H, int D, int L, int R, int causal, float scale,
+                      const int32_t *__restrict__ idx = nullptr, const uint8_t *__restrict__ mask = nullptr) {
     const int lane = threadIdx.x & 63;
     const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (unit >= (long)B * N * H) return;
@@ -230,7 +231,13 @@ attn_bwd_query_kernel(const typename T::storage *__restrict__ Q, const typename 
             if (j >= 0 && j < N && (!causal || j <= n)) r = j;
         } else if (t < S) {
             const int l = t - Wn;
-            if (!(causal && (((n >> l) & 1) == 0))) r = level_offset(N, l) + ((n >> l) ^ 1);
+            if (idx) {
+                // the caller's tables: an entry outside [0, M) or a set mask byte is a dead slot
+                const int e = idx[(size_t)n * L + l];
+                if (e >= 0 && e < M && !(mask && mask[(size_t)n * L + l])) r = e;
+            } else if (!(causal && (((n >> l) & 1) == 0))) {
+                r = level_offset(N, l) + ((n >> l) ^ 1);
+            }
         }
         row[c] = r;
         float s = -INFINITY, g = 0.f;
@@ -295,7 +302,7 @@ __global__ void __launch_bounds__(256)
 attn_bwd_key_kernel(const typename T::storage *__restrict__ Q, const typename T::storage *__restrict__ dO,
                     const float *__restrict__ Pw, const float *__restrict__ DS,
                     typename T::storage *__restrict__ dK, typename T::storage *__restrict__ dV, int B, int N, int M,
-                    int H, int D, int L, int R, int causal) {
+                    int H, int D, int L, int R, int causal, const int32_t *__restrict__ gather = nullptr) {
     const int lane = threadIdx.x & 63;
     const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (unit >= (long)B * M * H) return;
@@ -330,13 +337,20 @@ attn_bwd_key_kernel(const typename T::storage *__restrict__ Q, const typename T:
             for (int n = lo; n <= hi; ++n) add(n, row - n + R);
             if (L > 0) {
                 const int sib = row ^ 1;  // the query whose level-0 neighbour is this leaf
-                if (!causal || (sib & 1)) add(sib, Wn);
+                if (sib < N && (!causal || (sib & 1))) add(sib, Wn);
             }
         } else if (row < 2 * N - 2) {  // tree node below the root
             int lvl = 1;
             while (row >= level_offset(N, lvl + 1)) ++lvl;
             const int pidx = row - level_offset(N, lvl);
-            if (!causal || (pidx & 1) == 0) {
+            if (gather) {
+                // the caller's table: first of the 2^lvl queries that attend this node through their
+                // slot of level lvl, or -1 (what the reference's kernels read from it,
+                // ops/triton/sparse_attn.py:389-470); masked queries carry zero weights
+                const int first = gather[(size_t)row * 3];
+                if (lvl < L && first >= 0 && first + (1 << lvl) <= N)
+                    for (int n = first; n < first + (1 << lvl); ++n) add(n, Wn + lvl);
+            } else if (!causal || (pidx & 1) == 0) {
                 const int first = (pidx ^ 1) << lvl;
                 for (int n = first; n < first + (1 << lvl); ++n) add(n, Wn + lvl);
             }
@@ -594,9 +608,10 @@ static int attn_bwd_vec_try(const void *q, const void *k, const void *v, const v
 template <typename T>
 static int attn_bwd_typed(const void *q, const void *k, const void *v, const void *dout, void *dq, void *dk,
                           void *dv, float *ws_p, float *ws_ds, int B, int N, int M, int H, int D, int L, int R,
-                          int causal, hipStream_t st) {
+                          int causal, hipStream_t st, const int32_t *idx = nullptr, const uint8_t *mask = nullptr,
+                          const int32_t *gather = nullptr) {
     using S = typename T::storage;
-    {
+    if (!idx) {
         int rc = attn_bwd_vec_try<T>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal, st);
         if (rc != HSA_ERR_UNSUPPORTED) return rc;
     }
@@ -606,14 +621,14 @@ static int attn_bwd_typed(const void *q, const void *k, const void *v, const voi
     if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     attn_bwd_query_kernel<T><<<(unsigned)blocks, 256, 0, st>>>((const S *)q, (const S *)k, (const S *)v,
                                                                (const S *)dout, (S *)dq, ws_p, ws_ds, B, N, M, H, D,
-                                                               L, R, causal, scale);
+                                                               L, R, causal, scale, idx, mask);
     int rc = check_launch("attn_bwd_query_kernel");
     if (rc != HSA_OK) return rc;
     units = (long)B * M * H;
     blocks = (units + 3) / 4;
     if (blocks > 0x7fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     attn_bwd_key_kernel<T><<<(unsigned)blocks, 256, 0, st>>>((const S *)q, (const S *)dout, ws_p, ws_ds, (S *)dk,
-                                                             (S *)dv, B, N, M, H, D, L, R, causal);
+                                                             (S *)dv, B, N, M, H, D, L, R, causal, gather);
     return check_launch("attn_bwd_key_kernel");
 }
 
@@ -879,6 +894,29 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
         case HSA_BF16: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, causal ? 1 : 0, st);
     }
     return hsa::fail(HSA_ERR_INVALID, "unknown dtype %d", dtype);
+}
+
+int hsa_attn_bwd_tables(const void *q, const void *k, const void *v, const void *dout, const int32_t *idx,
+                        const uint8_t *mask, const int32_t *gather, void *dq, void *dk, void *dv, void *workspace,
+                        size_t workspace_bytes, int B, int N, int M, int H, int D, int L, int R, int causal, int dtype,
+                        void *stream) {
+    HSA_REQUIRE(q && k && v && dout && idx && gather && dq && dk && dv && workspace, "null pointer");
+    HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1 && L >= 0, "bad shape B=%d N=%d H=%d D=%d L=%d", B, N, H, D, L);
+    HSA_REQUIRE(M >= N, "key rows M=%d below the leaf count N=%d", M, N);
+    HSA_REQUIRE(R >= 0, "bad R=%d", R);
+    HSA_REQUIRE(dtype == HSA_F32 || dtype == HSA_F16 || dtype == HSA_BF16, "unknown dtype %d", dtype);
+    const size_t need = hsa::bwd_gather_ws_floats(B, N, H, L, R) * sizeof(float);
+    HSA_REQUIRE(workspace_bytes >= need, "workspace too small (%zu bytes, %zu needed)", workspace_bytes, need);
+    if (2 * R + 1 + L > 64 * hsa::BWD_MAX_CHUNKS)
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "2R+1+L = %d slots exceeds %d", 2 * R + 1 + L, 64 * hsa::BWD_MAX_CHUNKS);
+    hipStream_t st = (hipStream_t)stream;
+    float *ws_p = (float *)workspace, *ws_ds = ws_p + (size_t)B * N * H * (2 * R + 1 + L);
+    const int c = causal ? 1 : 0;
+    switch (dtype) {
+        case HSA_F32: return hsa::attn_bwd_typed<hsa::F32>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, c, st, idx, mask, gather);
+        case HSA_F16: return hsa::attn_bwd_typed<hsa::F16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, c, st, idx, mask, gather);
+        default: return hsa::attn_bwd_typed<hsa::BF16>(q, k, v, dout, dq, dk, dv, ws_p, ws_ds, B, N, M, H, D, L, R, c, st, idx, mask, gather);
+    }
 }
 
 int hsa_attn_bwd_saved_tune(int strip_blocks) {

@@ -368,6 +368,40 @@ def attention_backward(grad_out, Q, K, V, window_size: int, causal: bool, algo: 
     return dq, dk, dv
 
 
+def attention_backward_tables(grad_out, Q, K, V, idx_table, mask_table, gather_table, window_size: int):
+    """Gradients (dQ, dK, dV) of the span attention from the caller's own tables, as the
+    reference's backward computes them (hierarchical_attention/ops/functional.py:171-264): key
+    rows and dead slots from `idx_table` / `mask_table`, each node row's first attending query
+    from column 0 of `gather_table`; the window is causal when a mask table is given."""
+    _lib.require_gpu(grad_out, Q, K, V, idx_table, gather_table)
+    grad_out, Q, K, V = (t.contiguous() for t in (grad_out, Q, K, V))
+    B, N, H, D = Q.shape
+    M = K.shape[1]
+    assert idx_table.dim() == 2 and idx_table.shape[0] == N, "idx_table must be [N, L]"
+    L = idx_table.shape[1]
+    assert gather_table.dim() == 2 and gather_table.shape[1] >= 3 and gather_table.shape[0] >= min(M, 2 * N - 1), \
+        "gather_table must hold a row of three entries per key row"
+    idx = idx_table.to(torch.int32).contiguous()
+    gat = gather_table.to(torch.int32)[:, :3].contiguous()
+    m8 = None
+    if mask_table is not None:
+        assert mask_table.shape == idx_table.shape, "mask_table must have idx_table's shape"
+        m8 = mask_table.to(torch.bool).contiguous().view(torch.uint8)
+    R = int(window_size)
+    dq, dk, dv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
+    if Q.numel() == 0:
+        return dq, dk, dv
+    ws = torch.empty(2 * B * N * H * (2 * R + 1 + L) + 4, device=Q.device, dtype=torch.float32)
+    lib = _lib.lib()
+    with _lib.on_device(Q):
+        rc = lib.hsa_attn_bwd_tables(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(grad_out), _lib.ptr(idx),
+                                     _lib.ptr(m8), _lib.ptr(gat), _lib.ptr(dq), _lib.ptr(dk), _lib.ptr(dv),
+                                     _lib.ptr(ws), ws.numel() * 4, B, N, M, H, D, L, R,
+                                     int(mask_table is not None), _lib.dtype_code(Q), _lib.stream_of(Q))
+    _lib.check(rc, "hsa_attn_bwd_tables")
+    return dq, dk, dv
+
+
 class BuildParentNodesFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q_p, K_p, V_p, K_c, V_c):
@@ -425,15 +459,26 @@ class HierarchicalAttentionFunc(torch.autograd.Function):
                 ctx.save_for_backward(Q, K, V, out, lse)
                 return out
         out = attention_forward(Q, K, V, idx_table, mask_table, window_size)
-        ctx.save_for_backward(Q, K, V)
+        if canon is None and gather_table is not None:
+            # tables of the caller's own: the backward reads them like the reference's does
+            ctx.has_mask = mask_table is not None
+            ctx.save_for_backward(Q, K, V, idx_table, gather_table, *([mask_table] if ctx.has_mask else []))
+        else:
+            ctx.save_for_backward(Q, K, V)
         return out
 
     @staticmethod
     def backward(ctx, grad_output):
         if ctx.canonical is None:
-            raise NotImplementedError(
-                "hierarchical_attention backward needs the tables of build_tree_topology "
-                "(the reference's backward kernels make the same assumption through gather_table)")
+            if len(ctx.saved_tensors) < 5:
+                raise NotImplementedError(
+                    "hierarchical_attention backward with tables other than build_tree_topology's needs the "
+                    "gather_table that goes with them (the reference's backward kernels read it too)")
+            Q, K, V, idx_table, gather_table = ctx.saved_tensors[:5]
+            mask_table = ctx.saved_tensors[5] if ctx.has_mask else None
+            dq, dk, dv = attention_backward_tables(grad_output, Q, K, V, idx_table, mask_table, gather_table,
+                                                   ctx.window_size)
+            return dq, dk, dv, None, None, None, None
         if ctx.saved_state:
             Q, K, V, out, lse = ctx.saved_tensors
             if all(t.data_ptr() % 16 == 0 for t in (grad_output.contiguous(), Q, K, V, out)):

@@ -1214,7 +1214,7 @@ def test_attention_backward_long_sequence_upper_levels(causal):
     assert not tile[1][:, 2 * N - 2].any() and not tile[2][:, 2 * N - 2].any()
 
 
-def test_attention_backward_rejects_unknown_tables():
+def test_attention_backward_unknown_tables_need_their_gather_table():
     N = 16
     q, k, v = make_qkv(1, N, 1, 16, torch.float32, seed=1, M=40)
     idx = torch.randint(0, 40, (N, 4), dtype=torch.int32).to(DEV)
@@ -1222,6 +1222,50 @@ def test_attention_backward_rejects_unknown_tables():
     out = sa.hierarchical_attention(qd, k.to(DEV), v.to(DEV), idx, None, None, 2)
     with pytest.raises(NotImplementedError):
         out.sum().backward()
+
+
+@pytest.mark.parametrize("case", [(2, 32, 3, 16, 2, 70), (1, 64, 2, 64, 5, 127), (2, 16, 1, 20, 0, 31), (1, 128, 4, 32, 16, 300)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_backward_from_caller_tables(case, dtype, causal):
+    """Tables that are not build_tree_topology's (dead -1 slots, extra masked slots, node rows
+    whose gather entry says nobody attends them, more key rows than 2N-1): the backward reads the
+    caller's idx / mask / gather tables like the reference's does; against autograd through the
+    fp64 oracle, directly and through the autograd function."""
+    B, N, H, D, R, M = case
+    L = N.bit_length() - 1
+    q, k, v = make_qkv(B, N, H, D, dtype, seed=3 * N + R, M=M)
+    go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(R + 1)).to(dtype)
+    o = oracle.topology_tables(N, causal)
+    rng = np.random.default_rng(N + R)
+    idx = np.array(o["forward_idx"], dtype=np.int32).copy()
+    mask = np.array(o["forward_mask"], dtype=bool).copy() if causal else None
+    gather = np.array(o["backward_gather"], dtype=np.int32).copy()
+    idx[rng.random(idx.shape) < 0.15] = -1                     # dead slots
+    if causal:
+        mask |= rng.random(mask.shape) < 0.1                   # more masked slots
+    # a few node rows nobody attends: their queries' slots die, the gather entry says -1
+    for row in rng.choice(np.arange(N, 2 * N - 2), size=min(3, N - 2), replace=False):
+        lvl = 1
+        while row >= 2 * N - (N >> lvl):
+            lvl += 1
+        first = int(gather[row, 0])
+        if first >= 0:
+            idx[first:first + (1 << lvl), lvl] = -1
+        gather[row] = -1
+    if M > gather.shape[0]:
+        gather = np.concatenate([gather, -np.ones((M - gather.shape[0], 3), np.int32)])
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    oracle.attention_ref(qr, kr, vr, idx, mask, R).backward(go.double())
+    idx_d, gat_d = torch.from_numpy(idx).to(DEV), torch.from_numpy(gather).to(DEV)
+    mask_d = torch.from_numpy(mask).to(DEV) if causal else None
+    got = fn.attention_backward_tables(go.to(DEV), q.to(DEV), k.to(DEV), v.to(DEV), idx_d, mask_d, gat_d, R)
+    for name, g1, ref in zip(("dQ", "dK", "dV"), got, (qr.grad, kr.grad, vr.grad)):
+        _grad_close(g1, ref, dtype, "%s from the caller's tables, causal=%s" % (name, causal))
+    qa, ka, va = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    sa.hierarchical_attention(qa, ka, va, idx_d, gat_d, mask_d, R).backward(go.to(DEV))
+    for a, g1 in zip((qa.grad, ka.grad, va.grad), got):
+        assert torch.equal(a, g1)
 
 
 @pytest.mark.parametrize("shape", [(2, 1, 1, 8), (2, 5, 3, 16), (1, 64, 8, 64), (2, 16, 4, 128), (1, 7, 2, 20)])
