@@ -74,9 +74,12 @@ template <typename T, int D>
 struct BwdTile {
     using M_ = Mma<T>;
     static constexpr int KS = D / 32, NJ = D / 16, CPR = D / 8, RPI = 64 / CPR, NLD = TILE_Q / RPI;
-    static constexpr int PITCH = D * 2 + 16, BLK_BYTES = TILE_Q * PITCH;
+    // a block in LDS: rows back to back, the 16-byte pieces of row r at piece index p ^ swz(r)
+    // (conflict-free from both sides, see hsa_attn_tile.h); slots keep the size of a padded block
+    static constexpr int RB = D * 2, RPB = RB >= 256 ? 1 : 256 / RB, BLK_BYTES = TILE_Q * (RB + 16);
+    __device__ static __forceinline__ int swz(int row) { return (row / RPB) % CPR; }
 
-    int lane, r16, g, lrow, lchk;
+    int lane, r16, g, lrow, lchk, op_swz;
     unsigned char *lds;
     u32x4_t Pi[2];
 
@@ -86,6 +89,7 @@ struct BwdTile {
         g = lane >> 4;
         lrow = lane / CPR;
         lchk = lane % CPR;
+        op_swz = swz(r16);
         lds = wave_lds;
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
@@ -97,14 +101,17 @@ struct BwdTile {
     }
     // rows -> LDS -> operand pieces
     __device__ __forceinline__ void put(int slot, const u32x4_t (&raw)[NLD]) const {
-        unsigned char *reg = lds + slot * BLK_BYTES + lrow * PITCH + 16 * lchk;
+        unsigned char *reg = lds + slot * BLK_BYTES;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i) *reinterpret_cast<u32x4_t *>(reg + i * RPI * PITCH) = raw[i];
+        for (int i = 0; i < NLD; ++i) {
+            const int row = i * RPI + lrow;
+            *reinterpret_cast<u32x4_t *>(reg + row * RB + 16 * (lchk ^ swz(row))) = raw[i];
+        }
     }
     __device__ __forceinline__ void get(int slot, u32x4_t (&dst)[KS]) const {
-        const unsigned char *reg = lds + slot * BLK_BYTES + r16 * PITCH + 16 * g;
+        const unsigned char *reg = lds + slot * BLK_BYTES + r16 * RB;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const u32x4_t *>(reg + 64 * ks);
+        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const u32x4_t *>(reg + 16 * ((4 * ks + g) ^ op_swz));
     }
     // operand rows -> "lane = channel, regs = rows" form
     __device__ __forceinline__ void transpose(const u32x4_t (&op)[KS], u32x2_t (&dst)[NJ]) const {
@@ -118,17 +125,18 @@ struct BwdTile {
     // result tiles [channel, column] (this lane: column r16, channels 32ks+8g+4jj+i) -> packed
     // 16-bit pieces in LDS slot `slot`, one row per column
     __device__ __forceinline__ void put_result(int slot, const f32x4 (&t)[NJ], float mul) const {
-        unsigned char *reg = lds + slot * BLK_BYTES + r16 * PITCH + 16 * g;
+        unsigned char *reg = lds + slot * BLK_BYTES + r16 * RB;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const f32x4 a = t[2 * ks], b = t[2 * ks + 1];
-            *reinterpret_cast<u32x4_t *>(reg + 64 * ks) =
+            *reinterpret_cast<u32x4_t *>(reg + 16 * ((4 * ks + g) ^ op_swz)) =
                 u32x4_t{M_::pack(a[0] * mul, a[1] * mul), M_::pack(a[2] * mul, a[3] * mul),
                         M_::pack(b[0] * mul, b[1] * mul), M_::pack(b[2] * mul, b[3] * mul)};
         }
     }
     __device__ __forceinline__ u32x4_t get_row_piece(int slot, int i) const {
-        return *reinterpret_cast<const u32x4_t *>(lds + slot * BLK_BYTES + (i * RPI + lrow) * PITCH + 16 * lchk);
+        const int row = i * RPI + lrow;
+        return *reinterpret_cast<const u32x4_t *>(lds + slot * BLK_BYTES + row * RB + 16 * (lchk ^ swz(row)));
     }
 };
 

@@ -104,8 +104,15 @@ attn_tile_kernel(TileParams p) {
     constexpr int CPR = D / 8;                         // 16-byte pieces per head-row
     constexpr int RPI = 64 / CPR;                      // rows covered by one load instruction
     constexpr int NLD = TILE_Q / RPI;                  // load instructions per 16-row block
-    constexpr int PITCH = D * 2 + 16;                  // LDS row pitch in bytes (padding spreads banks)
-    constexpr int BLK_BYTES = TILE_Q * PITCH;          // one 16-row operand block in LDS
+    // One 16-row block in LDS: rows back to back (RB bytes each), the 16-byte pieces of row r
+    // stored at piece index p ^ swz(r).  The LDS serves a 16-byte access of 16 lanes per cycle
+    // from 64 four-byte banks: the row-major side (D/8 lanes per row, consecutive rows) then
+    // covers every bank once, and so does the operand side (lane = row, same piece), because
+    // rows that share banks get different swz values.  (A padded pitch of RB + 16 made only the
+    // operand side conflict-free: two rows of 144 bytes wrap around the 256 bytes of the banks.)
+    constexpr int RB = D * 2;
+    constexpr int RPB = RB >= 256 ? 1 : 256 / RB;      // rows per pass over the banks
+    constexpr int BLK_BYTES = TILE_Q * (RB + 16);      // a block's slot (the weights staging below uses the slack)
     constexpr int WAVE_LDS = 5 * BLK_BYTES;            // q, k, v, near-tree k, near-tree v
 
     __shared__ __align__(16) unsigned char smem[tile_max_wpb<D, NKL>() * WAVE_LDS];
@@ -255,15 +262,21 @@ attn_tile_kernel(TileParams p) {
         }
     };
     // LDS re-layout of one block: rows in, MFMA operand pieces out
+    auto swz = [](int row) { return (row / RPB) % CPR; };
+    const int op_swz = swz(r16);
     auto lds_put = [&](int slot, const u32x4_t (&raw)[NLD]) {
-        unsigned char *reg = lds + slot * BLK_BYTES + lrow * PITCH + 16 * lchk;
+        unsigned char *reg = lds + slot * BLK_BYTES;
 #pragma unroll
-        for (int i = 0; i < NLD; ++i) *reinterpret_cast<u32x4_t *>(reg + i * RPI * PITCH) = raw[i];
+        for (int i = 0; i < NLD; ++i) {
+            const int row = i * RPI + lrow;
+            *reinterpret_cast<u32x4_t *>(reg + row * RB + 16 * (lchk ^ swz(row))) = raw[i];
+        }
     };
     auto lds_get = [&](int slot, u32x4_t (&dst)[KS]) {
-        const unsigned char *reg = lds + slot * BLK_BYTES + r16 * PITCH + 16 * g;
+        const unsigned char *reg = lds + slot * BLK_BYTES + r16 * RB;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) dst[ks] = *reinterpret_cast<const u32x4_t *>(reg + 64 * ks);
+        for (int ks = 0; ks < KS; ++ks)
+            dst[ks] = *reinterpret_cast<const u32x4_t *>(reg + 16 * ((4 * ks + g) ^ op_swz));
     };
     auto transpose_v = [&](const u32x4_t (&op)[KS], u32x2_t (&dst)[NJ]) {
 #pragma unroll
@@ -474,7 +487,7 @@ attn_tile_kernel(TileParams p) {
 
         // O^T tiles: this lane ends with channels [32ks + 8g, +8) of query r16; through LDS
         // back to whole rows, then streaming stores (the output is not read again here)
-        unsigned char *oreg = lds + r16 * PITCH + 16 * g;
+        unsigned char *oreg = lds + r16 * RB;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             uint32_t w[4];
@@ -489,14 +502,14 @@ attn_tile_kernel(TileParams p) {
                 w[2 * jj] = M_::pack(o[0] * inv, o[1] * inv);
                 w[2 * jj + 1] = M_::pack(o[2] * inv, o[3] * inv);
             }
-            *reinterpret_cast<u32x4_t *>(oreg + 64 * ks) = u32x4_t{w[0], w[1], w[2], w[3]};
+            *reinterpret_cast<u32x4_t *>(oreg + 16 * ((4 * ks + g) ^ op_swz)) = u32x4_t{w[0], w[1], w[2], w[3]};
         }
         {
-            const unsigned char *src = lds + lrow * PITCH + 16 * lchk;
             uint16_t *optr = Ob + (size_t)(q0 + lrow) * rs;
 #pragma unroll
             for (int i = 0; i < NLD; ++i) {
-                const u32x4_t val = *reinterpret_cast<const u32x4_t *>(src + i * RPI * PITCH);
+                const int row = i * RPI + lrow;
+                const u32x4_t val = *reinterpret_cast<const u32x4_t *>(lds + row * RB + 16 * (lchk ^ swz(row)));
                 if constexpr ((HSA_TILE_NT & 32) != 0) *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = val;
                 else __builtin_nontemporal_store(val, reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs));
             }
