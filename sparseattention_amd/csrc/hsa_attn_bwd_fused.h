@@ -24,6 +24,8 @@
 // four blocks with the rows staged in registers: 56.0); with every load or every store removed
 // the same instruction stream takes 44 / 47 us, with both removed 36: the wavefront's own
 // instruction time is what is left to hide behind the memory system.
+// Requesting two blocks ahead (into the area whose operands have just left for the registers) is
+// slower: 52.4 us.
 // Strips of eight blocks where that still fills every wavefront slot: one neighbour's block per
 // 128 queries instead of per 64 (the far tree block and its partial rows change in the middle of
 // the strip, the leaf key blocks' accumulators just carry on).
