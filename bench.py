@@ -572,7 +572,7 @@ def main():
         min_total_ms=6.0))
     # the one-pass backward on saved forward state (opt-in: less traffic, more time), where it applies
     attn_bwd1_ms = None
-    if int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, _lib.HSA_BF16)) > 0:
+    if int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16)) > 0:
         saved = []
         for s in prob.sets:
             o_ = torch.empty_like(s["q"])

@@ -72,7 +72,7 @@ def _declare(lib):
     lib.hsa_build_parents_strided_bwd.restype = I
     lib.hsa_attn_fwd_lse.argtypes = [P] * 5 + [I] * 9 + [P]
     lib.hsa_attn_fwd_lse.restype = I
-    lib.hsa_attn_bwd_saved_workspace_bytes.argtypes = [I] * 8
+    lib.hsa_attn_bwd_saved_workspace_bytes.argtypes = [I] * 9
     lib.hsa_attn_bwd_saved_workspace_bytes.restype = ctypes.c_size_t
     lib.hsa_attn_bwd_saved.argtypes = [P] * 10 + [ctypes.c_size_t] + [I] * 9 + [P]
     lib.hsa_attn_bwd_saved.restype = I

@@ -42,13 +42,16 @@ int &bwd_fused_strip_knob();
 // Wavefronts per SIMD the fused pass is compiled for.
 constexpr int bwd_fused_waves(int D, bool causal) { return D <= 32 ? 2 : 1; }
 
-template <typename T, int D, bool CAUSAL, int SB>
+// NBW: 16-row blocks the window reaches to either side (window radius up to 16 NBW); two only with
+// the causal mask (without it four key blocks would wait for their last query block at a time).
+template <typename T, int D, bool CAUSAL, int SB, int NBW>
 __global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D, CAUSAL))))
 attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     using BT = BwdTile<T, D>;
     using M_ = Mma<T>;
     static_assert(SB == 4 || SB == 8, "a strip is one or two runs of four blocks (the 64 leaves under a level-6 node)");
-    constexpr int NBW = 1, FAR = BWD_STRIP;  // FAR: blocks that share the far tree block
+    static_assert(NBW == 1 || (NBW == 2 && CAUSAL), "window radius up to 16, or up to 32 with the causal mask");
+    constexpr int FAR = BWD_STRIP;  // blocks that share the far tree block
     constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD, CPR = BT::CPR;
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
     constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
@@ -63,8 +66,10 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     // is free at that moment.
     constexpr int RB = 2 * D, ARR = TILE_Q * RB, STG = 6 * ARR, RPB = 256 / RB;
     __shared__ __align__(16) unsigned char stage_mem[BWD_WPB * 2 * STG];
-    // dK^T / dV^T of the key blocks that wait for the next query block: one when causal, two otherwise
-    constexpr int NPARK = CAUSAL ? 1 : 2;
+    // dK^T / dV^T of the key blocks that wait for their remaining query blocks: NBW when causal,
+    // 2 NBW otherwise; the slot of key block j is j mod NPARK
+    constexpr int NPARK = CAUSAL ? NBW : 2 * NBW;
+    static_assert(NPARK <= 2, "the slot is taken from the block's parity");
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * BWD_WPB + wave;
@@ -287,7 +292,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     // everything the first block needs is requested before anything is consumed
     u32x4_t Kc[NKB][KS], Vc[NKB][KS];
     u32x4_t rKu[NLD], rVu[NLD];  // the far block's rows on their way
-    float halo_lse4[4];
+    float halo_lse4[NBW][4];
     using Area0 = std::integral_constant<int, 0>;
     using Area1 = std::integral_constant<int, STG>;
     const bool left_halo = !CAUSAL && blk0 > 0, right_halo = blk0 + SB < NB;  // uniform
@@ -299,7 +304,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             load_block(Kb, leaf_row0(blk0 - NBW + c), rKh[c]);
             load_block(Vb, leaf_row0(blk0 - NBW + c), rVh[c]);
         }
-        if constexpr (!CAUSAL) request_halo_dma(STG, blk0 - 1, halo_lse4);
+        if constexpr (!CAUSAL) request_halo_dma(STG, blk0 - 1, halo_lse4[0]);
         request_dma(0, blk0);
 #pragma unroll
         for (int c = 0; c + 1 < NKL; ++c) {
@@ -316,7 +321,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
         wait_vmem_all_but<6 * NLD>();  // everything older than the first block's transfers
-        if (left_halo) halo_contrib(Area1{}, halo_lse4, blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
+        if (left_halo) halo_contrib(Area1{}, halo_lse4[0], blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
         park_put(0, tk, tv);
     }
     // partial rows of the far block, summed over a run of four blocks
@@ -348,16 +353,19 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         // so the wait names how many younger operations may still be in flight: the transfers
         // just requested plus the previous block's stores, which follow this block's request in
         // program order.  Only stores that are certainly issued are counted (dQ: NLD; the finished
-        // leaf key block: 2 NLD from the strip's second block on; near tree rows: 2 NLD, some
+        // leaf key block: 2 NLD from block NBW of the strip on; near tree rows: 2 NLD, some
         // lane always has a row); counting too few only waits longer.
         if (it + 1 < SB) {
             request_dma((PAR ^ 1) * STG, blk + 1);
             if (it == 0) wait_vmem_all_but<6 * NLD>();
-            else if (it == 1) wait_vmem_all_but<6 * NLD + 3 * NLD>();
+            else if (it <= NBW) wait_vmem_all_but<6 * NLD + 3 * NLD>();
             else wait_vmem_all_but<6 * NLD + 5 * NLD>();
         } else {
-            request_halo_dma((PAR ^ 1) * STG, blk0 + SB, halo_lse4);
-            wait_vmem_all_but<3 * NLD + 4 + 5 * NLD>();  // SB >= 4: the block before stored all of the above
+            // the neighbour's query blocks, three staged blocks each, into the halves of the area
+#pragma unroll
+            for (int hq = 0; hq < NBW; ++hq) request_halo_dma((PAR ^ 1) * STG + hq * 3 * ARR, blk0 + SB + hq, halo_lse4[hq]);
+            static_assert(SB - 2 >= NBW, "the block before the last stored all of the above");
+            wait_vmem_all_but<NBW * (3 * NLD + 4) + 5 * NLD>();
         }
         if constexpr (KS == 2)
             lds_read16_6x2<PAR * STG, ARR>(opa0, opa1, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
@@ -490,7 +498,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             const int SLOT = ((PAR + NBW + c) & 1) & (NPARK - 1);      // j % NPARK (NBW + it + c has j's parity)
             if (j >= 0 && j < SB) {
                 f32x4 tk[NJ], tv[NJ];
-                const bool fresh = c == NKL - 1 && (CAUSAL || j > 0);  // nobody has contributed yet
+                const bool fresh = c == NKL - 1 && (CAUSAL || j >= NBW);  // nobody has contributed yet
                 if (fresh) {
 #pragma unroll
                     for (int jj = 0; jj < NJ; ++jj) { tk[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[jj] = f32x4{0.f, 0.f, 0.f, 0.f}; }
@@ -608,15 +616,26 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         }
     }
 
-    // the strip's last key block: the query block after the strip reaches it (the block sits in
-    // the first operand slot after the last slide)
+    // the strip's last NBW key blocks: the query blocks after the strip reach them (their operands
+    // sit in the first slots after the last slide; the neighbour's block hq reaches the last
+    // NBW - hq of them)
     {
-        static_assert(SB % 2 == 0, "the neighbour's block is staged in the first area");
-        f32x4 tk[NJ], tv[NJ];
-        park_get(((SB - 1) & 1) & (NPARK - 1), tk, tv);
+        static_assert(SB % 2 == 0, "the neighbour's blocks are staged in the first area");
         wait_vmem_all_but<0>();
-        if (right_halo) halo_contrib(Area0{}, halo_lse4, blk0 + SB, Kc[0], Vc[0], blk0 + SB - 1, tk, tv);
-        store_key_block(blk0 + SB - 1, tk, tv);
+#pragma unroll
+        for (int e = 0; e < NBW; ++e) {  // key block blk0 + SB - NBW + e, operands in slot e
+            const int j = SB - NBW + e;
+            f32x4 tk[NJ], tv[NJ];
+            park_get((j & 1) & (NPARK - 1), tk, tv);
+#pragma unroll
+            for (int hq = 0; hq <= e; ++hq) {
+                if (blk0 + SB + hq < NB) {  // uniform
+                    if (hq == 0) halo_contrib(Area0{}, halo_lse4[0], blk0 + SB, Kc[e], Vc[e], blk0 + j, tk, tv);
+                    else halo_contrib(std::integral_constant<int, 3 * ARR>{}, halo_lse4[NBW - 1], blk0 + SB + hq, Kc[e], Vc[e], blk0 + j, tk, tv);
+                }
+            }
+            store_key_block(blk0 + j, tk, tv);
+        }
     }
 }
 
@@ -643,15 +662,21 @@ int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t 
         const bool fills = (long)(fp.t.n_units / 8) >= 1024; /* one wavefront per SIMD on 256 CUs */       \
         const int knob = bwd_fused_strip_knob();                                                            \
         const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D == 64 && fills))) ? 8 : 4;             \
+        const int nbw = fp.t.R > TILE_Q ? 2 : 1;                                                            \
+        if (nbw == 2 && !causal) return fail(HSA_ERR_UNSUPPORTED, "one-pass backward: window radius above 16 needs the causal mask"); \
         q.t.n_units = fp.t.n_units / sb;                                                                    \
         q.t.red_lg_sb = sb == 8 ? 3 : 2;                                                                    \
         const int nwg = (q.t.n_units + BWD_WPB - 1) / BWD_WPB;                                              \
-        if (sb == 8) {                                                                                      \
-            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 8><<<nwg, BWD_WPB * 64, 0, st>>>(q);         \
-            else attn_bwd_tile_fused_kernel<T, D, false, 8><<<nwg, BWD_WPB * 64, 0, st>>>(q);               \
+        const dim3 grid(nwg), block(BWD_WPB * 64);                                                          \
+        if (nbw == 2) {                                                                                     \
+            if (sb == 8) attn_bwd_tile_fused_kernel<T, D, true, 8, 2><<<grid, block, 0, st>>>(q);           \
+            else attn_bwd_tile_fused_kernel<T, D, true, 4, 2><<<grid, block, 0, st>>>(q);                   \
+        } else if (sb == 8) {                                                                               \
+            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 8, 1><<<grid, block, 0, st>>>(q);            \
+            else attn_bwd_tile_fused_kernel<T, D, false, 8, 1><<<grid, block, 0, st>>>(q);                  \
         } else {                                                                                            \
-            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 4><<<nwg, BWD_WPB * 64, 0, st>>>(q);         \
-            else attn_bwd_tile_fused_kernel<T, D, false, 4><<<nwg, BWD_WPB * 64, 0, st>>>(q);               \
+            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 4, 1><<<grid, block, 0, st>>>(q);            \
+            else attn_bwd_tile_fused_kernel<T, D, false, 4, 1><<<grid, block, 0, st>>>(q);                  \
         }                                                                                                   \
         int rc = check_launch("attn_bwd_tile_fused_kernel");                                                \
         if (rc != HSA_OK || q.t.red_wgs == 0) return rc;                                                    \

@@ -98,8 +98,9 @@ static int tile_launch_wide_weights(const TileParams &p, int wpb, hipStream_t st
             case 1: return tile_launch_lse<T, D, 0, true>(p, sb, wpb, st);                      \
             case 2: return tile_launch_lse<T, D, 1, false>(p, sb, wpb, st);                     \
             case 3: return tile_launch_lse<T, D, 1, true>(p, sb, wpb, st);                      \
+            case 5: return tile_launch_lse<T, D, 2, true>(p, sb, wpb, st);                      \
         }                                                                                       \
-        return fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output is built for window radius up to 16"); \
+        return fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output is built for window radius up to 16, or 32 with the causal mask"); \
     }                                                                                           \
     template <>                                                                                 \
     int attn_tile_weights_launch_td<T, D>(const TileParams &p, int nbw, bool causal, int wpb,  \

@@ -755,11 +755,12 @@ int &bwd_fused_strip_knob() {
 template <typename T, int D>
 int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
 
-static bool attn_bwd_fused_eligible(int N, int M, int D, int L, int R, int dtype) {
+static bool attn_bwd_fused_eligible(int N, int M, int D, int L, int R, int dtype, int causal) {
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
     if (D != 32 && D != 64) return false;
     if (N < TILE_Q * BWD_STRIP || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
-    return R <= TILE_Q;
+    // one block of neighbours to either side, or two with the causal mask
+    return R <= TILE_Q || (R <= 2 * TILE_Q && causal != 0);
 }
 // partial rows of dK and dV for levels >= 6, laid out like the two-pass workspace without its
 // statistics
@@ -926,8 +927,8 @@ int hsa_attn_bwd_saved_tune(int strip_blocks) {
     return HSA_OK;
 }
 
-size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int dtype) {
-    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype)) return 0;
+size_t hsa_attn_bwd_saved_workspace_bytes(int B, int N, int M, int H, int D, int L, int R, int causal, int dtype) {
+    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype, causal)) return 0;
     return hsa::bwd_fused_ws_floats(B, N, H, D, L) * sizeof(float);
 }
 
@@ -939,13 +940,14 @@ int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *
     HSA_REQUIRE(hsa::ilog2_exact(N) == L, "canonical table needs L == log2 N (N=%d L=%d)", N, L);
     HSA_REQUIRE(M >= 2 * N - 1, "canonical table needs M >= 2N-1 (N=%d M=%d)", N, M);
     HSA_REQUIRE(R >= 0, "bad R=%d", R);
-    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype))
-        return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward not available for N=%d D=%d L=%d R=%d dtype=%d "
-                         "(16-bit types, 32 or 64 channels per head, radius up to 16, at least 64 leaves)", N, D, L, R, dtype);
+    if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype, causal))
+        return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward not available for N=%d D=%d L=%d R=%d causal=%d dtype=%d "
+                         "(16-bit types, 32 or 64 channels per head, radius up to 16, or up to 32 with the causal mask, "
+                         "at least 64 leaves)", N, D, L, R, causal ? 1 : 0, dtype);
     const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout |
                            (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)workspace) & 15) == 0;
     if (!aligned) return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward needs 16-byte aligned tensors");
-    HSA_REQUIRE(workspace_bytes >= hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, dtype),
+    HSA_REQUIRE(workspace_bytes >= hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, causal, dtype),
                 "workspace too small (%zu bytes)", workspace_bytes);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == HSA_BF16)

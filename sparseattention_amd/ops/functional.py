@@ -107,7 +107,7 @@ def attention_forward(Q, K, V, idx_table, mask_table=None, window_size: int = 16
     return (out, weights) if return_weights else out
 
 
-def saved_state_backward_available(Q, K, window_size: int) -> bool:
+def saved_state_backward_available(Q, K, window_size: int, causal: bool = True) -> bool:
     """Whether the one-pass backward (hsa_attn_bwd_saved) takes this problem on the canonical
     tables: then the forward should also keep its log-sum-exp (`attention_forward_lse`)."""
     if not Q.is_cuda or Q.dim() != 4:
@@ -116,7 +116,8 @@ def saved_state_backward_available(Q, K, window_size: int) -> bool:
     if N < 1 or (N & (N - 1)) or Q.dtype not in (torch.float16, torch.bfloat16):
         return False
     return int(_lib.lib().hsa_attn_bwd_saved_workspace_bytes(B, N, K.shape[1], H, D, N.bit_length() - 1,
-                                                            int(window_size), _lib.dtype_code(Q))) > 0
+                                                            int(window_size), int(bool(causal)),
+                                                            _lib.dtype_code(Q))) > 0
 
 
 def attention_forward_lse(Q, K, V, window_size: int, causal: bool):
@@ -151,7 +152,7 @@ def attention_backward_saved(grad_out, Q, K, V, out, lse, window_size: int, caus
     assert lse.shape == (B, N, H) and lse.dtype == torch.float32 and out.shape == Q.shape
     dq, dk, dv = torch.empty_like(Q), torch.empty_like(K), torch.empty_like(V)
     lib = _lib.lib()
-    nbytes = int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, _lib.dtype_code(Q)))
+    nbytes = int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, int(bool(causal)), _lib.dtype_code(Q)))
     ws = torch.empty((max(nbytes, 4) + 3) // 4, device=Q.device, dtype=torch.float32)
     with _lib.on_device(Q):
         rc = lib.hsa_attn_bwd_saved(_lib.ptr(Q), _lib.ptr(K), _lib.ptr(V), _lib.ptr(out), _lib.ptr(lse),
@@ -428,7 +429,7 @@ one_pass_backward = None
 
 
 def _use_one_pass(Q, K, window_size, causal) -> bool:
-    if one_pass_backward is False or not saved_state_backward_available(Q, K, window_size):
+    if one_pass_backward is False or not saved_state_backward_available(Q, K, window_size, causal):
         return False
     return True
 

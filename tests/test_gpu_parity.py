@@ -1073,7 +1073,9 @@ def test_attention_backward_wide_window_128_channels_both_formulations(dtype, ca
 
 
 SAVED_BWD_CASES = [(2, 64, 2, 64, 16), (1, 128, 3, 64, 5), (2, 256, 4, 32, 16), (1, 512, 2, 64, 0), (2, 1024, 8, 64, 16),
-                   (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1), (1, 128, 1, 32, 16), (1, 4096, 3, 64, 13)]
+                   (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1), (1, 128, 1, 32, 16), (1, 4096, 3, 64, 13),
+                   # window radius 17..32: two blocks of neighbours, with the causal mask only
+                   (2, 64, 2, 64, 32), (1, 128, 3, 64, 17), (2, 256, 2, 32, 32), (1, 1024, 4, 64, 25), (1, 2048, 1, 32, 20)]
 
 
 @pytest.mark.parametrize("case", SAVED_BWD_CASES)
@@ -1086,6 +1088,10 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
     log-sum-exp against the oracle's logits.  One strip (no neighbours), first / last strips and
     inner strips all occur."""
     B, N, H, D, R = case
+    if R > 16 and not causal:
+        qz = torch.zeros(B, N, H, D, dtype=dtype, device=DEV)
+        assert not fn.saved_state_backward_available(qz, torch.zeros(B, 2 * N - 1, H, D, dtype=dtype, device=DEV), R, False)
+        return
     q, k, v = make_qkv(B, N, H, D, dtype, seed=5 * N + R)
     go = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(N + R)).to(dtype)
     o = oracle.topology_tables(N, causal)
@@ -1094,7 +1100,7 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
                                             return_weights=True)
     want_out.backward(go.double())
     qd, kd, vd, gd = q.to(DEV), k.to(DEV), v.to(DEV), go.to(DEV)
-    assert fn.saved_state_backward_available(qd, kd, R)
+    assert fn.saved_state_backward_available(qd, kd, R, causal)
     out, lse = fn.attention_forward_lse(qd, kd, vd, R, causal)
     t = sa.build_tree_topology(N, causal, device=DEV)
     plain = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"] if causal else None, R)
@@ -1151,14 +1157,15 @@ def test_attention_backward_saved_state_limits():
     q = torch.zeros(1, 64, 2, 64, dtype=torch.bfloat16, device=DEV)
     k = torch.zeros(1, 127, 2, 64, dtype=torch.bfloat16, device=DEV)
     assert fn.saved_state_backward_available(q, k, 16)
-    assert not fn.saved_state_backward_available(q, k, 17)                      # radius above one block
+    assert not fn.saved_state_backward_available(q, k, 17, False)               # radius above one block without the mask
+    assert fn.saved_state_backward_available(q, k, 32, True) and not fn.saved_state_backward_available(q, k, 33, True)
     assert not fn.saved_state_backward_available(q.float(), k.float(), 16)      # fp32
     assert not fn.saved_state_backward_available(q[:, :32], k[:, :63], 16)      # fewer than 64 leaves
     q128 = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device=DEV)
     assert not fn.saved_state_backward_available(q128, torch.zeros(1, 127, 2, 128, dtype=torch.bfloat16, device=DEV), 16)
     lib = _lib.lib()
     d = _lib.ptr(q)
-    rc = lib.hsa_attn_bwd_saved(d, d, d, d, d, d, d, d, d, d, 1 << 20, 1, 64, 127, 2, 64, 6, 17, 1, 2, _lib.stream_of(q))
+    rc = lib.hsa_attn_bwd_saved(d, d, d, d, d, d, d, d, d, d, 1 << 20, 1, 64, 127, 2, 64, 6, 17, 0, 2, _lib.stream_of(q))
     assert rc == -95 and b"one-pass" in lib.hsa_last_error()
 
 
