@@ -310,14 +310,13 @@ int hsa_attn_bwd(const void *q, const void *k, const void *v, const void *dout, 
  * neighbouring strips' queries add is rebuilt from their Q, dO rows, lse and delta = <dO, out>),
  * so Q, dO, K, V are read once instead of twice.  Same results as hsa_attn_bwd to the rounding of
  * the element type; deterministic.  Canonical tables only; fp16 / bf16, 32 or 64 channels per
- * head, window radius up to 16 (up to 32 with the causal mask), N >= 64, 16-byte aligned tensors:
- * anything else returns
+ * head (128 with the causal mask), window radius up to 16 (up to 32 with the causal mask), N >= 64,
+ * 16-byte aligned tensors: anything else returns
  * HSA_ERR_UNSUPPORTED (hsa_attn_bwd_saved_workspace_bytes returns 0) and the caller uses
  * hsa_attn_bwd.  workspace: hsa_attn_bwd_saved_workspace_bytes(...) bytes, written before read.
  *
  * hsa_attn_fwd_lse: hsa_attn_fwd on the canonical tables that also writes lse (a variant of the
- * 16-bit tile kernel, built for the shapes hsa_attn_bwd_saved takes: up to 64 channels per head,
- * window radius up to 16, or up to 32 with the causal mask; HSA_ERR_UNSUPPORTED otherwise, nothing
+ * 16-bit tile kernel, built for window radius up to 16, or up to 32 with the causal mask; HSA_ERR_UNSUPPORTED otherwise, nothing
  * launched).
  */
 int hsa_attn_fwd_lse(const void *q, const void *k, const void *v, void *out, float *lse, int B, int N, int M,

@@ -90,7 +90,7 @@ int hsa_attn_fwd_lse(const void *q, const void *k, const void *v, void *out, flo
     HSA_REQUIRE(q && k && v && out && lse, "null pointer");
     HSA_REQUIRE(B >= 1 && N >= 1 && H >= 1 && D >= 1, "bad shape B=%d N=%d H=%d D=%d", B, N, H, D);
     HSA_REQUIRE(L >= 0 && R >= 0, "bad L=%d R=%d", L, R);
-    if ((dtype != HSA_F16 && dtype != HSA_BF16) || D > 64 || R > (causal ? 32 : 16) ||
+    if ((dtype != HSA_F16 && dtype != HSA_BF16) || R > (causal ? 32 : 16) ||
         !hsa::attn_tile_eligible(N, M, H, D, L, R, dtype, true, false, causal != 0) ||
         ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0))
         return hsa::fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output comes from the 16-bit tile kernel only "

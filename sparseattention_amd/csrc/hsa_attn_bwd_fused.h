@@ -44,10 +44,21 @@ constexpr int bwd_fused_waves(int D, bool causal) { return D <= 32 ? 2 : 1; }
 
 // NBW: 16-row blocks the window reaches to either side (window radius up to 16 NBW); two only with
 // the causal mask (without it four key blocks would wait for their last query block at a time).
-template <typename T, int D, bool CAUSAL, int SB, int NBW>
-__global__ void __launch_bounds__(BWD_WPB * 64) __attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D, CAUSAL))))
+//
+// SPLIT = 2 (heads of 128 channels): a wavefront cannot hold the accumulators of 128 channels, so
+// two wavefronts share a (batch, strip, head): each owns 64 of the channels (its half of every
+// row, its half of dQ, dK, dV) and computes its half of every dot product over the channels; the
+// halves of the score and dP tiles are exchanged through LDS and added (both wavefronts then hold
+// bit-identical sums, so their softmax statistics agree).  The two are a workgroup of their own,
+// so that its barrier couples nobody else.
+template <typename T, int D, bool CAUSAL, int SB, int NBW, int SPLIT>
+__global__ void __launch_bounds__((SPLIT == 2 ? 2 : BWD_WPB) * 64)
+__attribute__((amdgpu_waves_per_eu(bwd_fused_waves(D / SPLIT, CAUSAL))))
 attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
-    using BT = BwdTile<T, D>;
+    static_assert(SPLIT == 1 || SPLIT == 2, "one wavefront per head, or two");
+    constexpr int HD = D / SPLIT;                       // channels a wavefront owns
+    constexpr int WPB = SPLIT == 2 ? 2 : BWD_WPB;       // wavefronts per workgroup
+    using BT = BwdTile<T, HD>;
     using M_ = Mma<T>;
     static_assert(SB == 4 || SB == 8, "a strip is one or two runs of four blocks (the 64 leaves under a level-6 node)");
     static_assert(NBW == 1 || (NBW == 2 && CAUSAL), "window radius up to 16, or up to 32 with the causal mask");
@@ -55,29 +66,40 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD, CPR = BT::CPR;
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;
     constexpr int NKB = NKL + 2;  // leaf blocks, near tree block, far tree block
-    constexpr int LDS_SLOTS = 4;
+    constexpr int LDS_SLOTS = 2;
     const BwdTileParams &p = fp.t;
-    __shared__ __align__(16) unsigned char smem[BWD_WPB * LDS_SLOTS * BT::BLK_BYTES];
-    __shared__ __align__(16) float carry_mem[BWD_WPB * 2 * D];
-    __shared__ __align__(16) float delta_mem[BWD_WPB * TILE_Q];
+    __shared__ __align__(16) unsigned char smem[WPB * LDS_SLOTS * BT::BLK_BYTES];
+    __shared__ __align__(16) float carry_mem[WPB * 2 * HD];
+    __shared__ __align__(16) float delta_mem[WPB * TILE_Q];
     // A block's rows (Q, dO, entering leaf K / V, near tree K / V: six 16-row blocks) go from
-    // global memory straight into one of two staging areas per wavefront, unpadded, with the
-    // pieces of each row permuted (hsa_lds_dma.h); the neighbour's query block uses the area that
-    // is free at that moment.
-    constexpr int RB = 2 * D, ARR = TILE_Q * RB, STG = 6 * ARR, RPB = 256 / RB;
-    __shared__ __align__(16) unsigned char stage_mem[BWD_WPB * 2 * STG];
+    // global memory straight into the wavefront's staging area, unpadded, with the pieces of each
+    // row permuted (hsa_lds_dma.h).  One area is enough: a block's operands leave it for the
+    // registers at the top of its iteration, and the next block's rows are requested right after.
+    // The neighbour's query blocks after the strip (three staged blocks each) use the area once
+    // the last block has left it; the one before the strip (no causal mask) has three blocks of
+    // its own behind the area.
+    constexpr int RB = 2 * HD, ARR = TILE_Q * RB, STG = 6 * ARR, RPB = 256 / RB;
+    constexpr int WAVE_STG = STG + (CAUSAL ? 0 : 3 * ARR);
+    __shared__ __align__(16) unsigned char stage_mem[WPB * WAVE_STG];
+    // exchange of partial tiles between the two wavefronts of a head: two slots per wavefront,
+    // used in turn, of XF4 16-byte values per lane
+    constexpr int XF4 = 2 * NKB;
+    __shared__ __align__(16) f32x4 xch_mem[SPLIT == 2 ? 2 * 2 * XF4 * 64 : 1];
     // dK^T / dV^T of the key blocks that wait for their remaining query blocks: NBW when causal,
     // 2 NBW otherwise; the slot of key block j is j mod NPARK
     constexpr int NPARK = CAUSAL ? NBW : 2 * NBW;
     static_assert(NPARK <= 2, "the slot is taken from the block's parity");
 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int unit = bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * BWD_WPB + wave;
+    // SPLIT == 2: the workgroup is one unit, its wavefronts the two channel halves
+    const int unit = SPLIT == 2 ? bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x)
+                                : bwd_xcd_remap((int)blockIdx.x, (int)gridDim.x) * WPB + wave;
+    const int half = SPLIT == 2 ? wave : 0;
     if (unit >= p.n_units) return;
     BT bt;
     bt.init(smem + wave * LDS_SLOTS * BT::BLK_BYTES);
     const int r16 = bt.r16, g = bt.g, lrow = bt.lrow, lchk = bt.lchk;
-    float *carry = carry_mem + wave * 2 * D;
+    float *carry = carry_mem + wave * 2 * HD;
     float *delta_lds = delta_mem + wave * TILE_Q;
     // slots are compile-time constants: plain registers
     f32x4 PK[NPARK][NJ], PV[NPARK][NJ];
@@ -97,15 +119,37 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     const int b = unit / (H * NS);
     const int blk0 = strip * SB;
     const size_t rs = (size_t)H * D;
-    const uint16_t *Q0 = p.q + ((size_t)b * N * H + h) * D, *G0 = p.dout + ((size_t)b * N * H + h) * D;
-    const uint16_t *O0 = fp.out + ((size_t)b * N * H + h) * D;
-    const uint16_t *K0 = p.k + ((size_t)b * p.M * H + h) * D, *V0 = p.v + ((size_t)b * p.M * H + h) * D;
+    const size_t qo = ((size_t)b * N * H + h) * D + half * HD, ko = ((size_t)b * p.M * H + h) * D + half * HD;
+    const uint16_t *Q0 = p.q + qo, *G0 = p.dout + qo, *O0 = fp.out + qo;
+    const uint16_t *K0 = p.k + ko, *V0 = p.v + ko;
     const uint16_t *Kb = K0 + 8 * lchk, *Vb = V0 + 8 * lchk;
-    uint16_t *dKb = p.dk + ((size_t)b * p.M * H + h) * D + 8 * lchk;
-    uint16_t *dVb = p.dv + ((size_t)b * p.M * H + h) * D + 8 * lchk;
+    uint16_t *dKb = p.dk + ko + 8 * lchk;
+    uint16_t *dVb = p.dv + ko + 8 * lchk;
+    // key / value blocks in operand form: the leaf blocks a query block reaches (they slide along
+    // the strip), the near tree block, the far tree block
+    u32x4_t Kc[NKB][KS], Vc[NKB][KS];
+    // adds the other wavefront's partial tiles to n of this wavefront's (SPLIT == 2 only; both
+    // wavefronts of the workgroup get here the same number of times)
+    int xslot = 0;
+    auto exchange = [&](auto n_tag, f32x4 *vals) {
+        constexpr int NX = decltype(n_tag)::value;
+        static_assert(NX <= XF4, "more values than a slot holds");
+        if constexpr (SPLIT == 2) {
+            f32x4 *mine = xch_mem + ((wave * 2 + xslot) * XF4) * 64 + bt.lane;
+            const f32x4 *other = xch_mem + (((wave ^ 1) * 2 + xslot) * XF4) * 64 + bt.lane;
+#pragma unroll
+            for (int k = 0; k < NX; ++k) mine[k * 64] = vals[k];
+            lds_only_barrier();
+#pragma unroll
+            for (int k = 0; k < NX; ++k) vals[k] += other[k * 64];
+            // the slot is written again two exchanges on, after the barrier of the next one,
+            // which the other wavefront passes only with these reads behind it
+            xslot ^= 1;
+        }
+    };
     // staging: the piece of its row a lane fetches (in elements), the lane's operand addresses for
     // the two contraction steps, and its own 16 bytes of a transfer
-    const uint32_t stg_base = lds_address(stage_mem) + wave * 2 * STG;
+    const uint32_t stg_base = lds_address(stage_mem) + wave * WAVE_STG;
     int pc8[NLD];
 #pragma unroll
     for (int i = 0; i < NLD; ++i) pc8[i] = 8 * (lchk ^ (((i * RPI + lrow) / RPB) % CPR));
@@ -208,18 +252,23 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         dma_block(O0, qb * TILE_Q, dst + 2 * ARR);
     };
 
-    // contribution of one query block (operands Qf/Gf, their transposes, the queries' lse and
-    // delta in the "regs = queries 4g+i" form) to the leaf key block kb (operands Kf/Vf)
-    auto leaf_contrib = [&](const u32x4_t (&Qf)[KS], const u32x4_t (&Gf)[KS], const u32x2_t (&QT)[NJ],
-                            const u32x2_t (&GT)[NJ], const float (&lse4)[4], const float (&del4)[4],
-                            const u32x4_t (&Kf)[KS], const u32x4_t (&Vf)[KS], int qb, int kb, f32x4 (&tk)[NJ],
-                            f32x4 (&tv)[NJ]) {
-        f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+    // One query block (operands Qf / Gf) against one leaf key block (operands Kf / Vf), second
+    // orientation: this wavefront's part of S[query 4g+i, key r16] and dP[query, key] ...
+    auto leaf_scores = [&](const u32x4_t (&Qf)[KS], const u32x4_t (&Gf)[KS], const u32x4_t (&Kf)[KS],
+                           const u32x4_t (&Vf)[KS], f32x4 &a, f32x4 &d) {
+        a = f32x4{0.f, 0.f, 0.f, 0.f};
+        d = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            a = M_::k32(Qf[ks], Kf[ks], a);  // S[query 4g+i of block qb, key r16 of block kb]
+            a = M_::k32(Qf[ks], Kf[ks], a);
             d = M_::k32(Gf[ks], Vf[ks], d);
         }
+    };
+    // ... and, from the complete tiles, the block's contribution to dK^T / dV^T of key block kb (the
+    // queries' transposed operands, their lse and delta in the "regs = queries 4g+i" form)
+    auto leaf_apply = [&](const f32x4 &a, const f32x4 &d, const u32x2_t (&QT)[NJ], const u32x2_t (&GT)[NJ],
+                          const float (&lse4)[4], const float (&del4)[4], int qb, int kb, f32x4 (&tk)[NJ],
+                          f32x4 (&tv)[NJ]) {
         float pp[4], ds[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -240,11 +289,13 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             tv[j] = M_::k16(GT[j], pk, tv[j]);
         }
     };
-    // contribution of a neighbouring strip's staged query block (area offset as a compile-time
-    // tag) to one of this strip's key blocks
-    auto halo_contrib = [&](auto area_tag, const float (&lse4)[4], int qb, const u32x4_t (&Kf)[KS],
-                            const u32x4_t (&Vf)[KS], int kb, f32x4 (&tk)[NJ], f32x4 (&tv)[NJ]) {
+    // A neighbouring strip's staged query block qb (area offset as a compile-time tag) against NK
+    // of this strip's key blocks (operand slots e0 .. e0 + NK - 1, key blocks kb0 ...): rebuilt
+    // from the block's Q and dO rows, its log-sum-exp and delta[q] = <dO[q], O[q]>.
+    auto halo_block = [&](auto area_tag, auto nk_tag, const float (&lse4)[4], int qb, int e0, int kb0,
+                          f32x4 (*tk)[NJ], f32x4 (*tv)[NJ]) {
         constexpr int OFF = decltype(area_tag)::value;
+        constexpr int NK = decltype(nk_tag)::value;
         u32x4_t Qf[KS], Gf[KS], gw[NLD], ow[NLD];
         if constexpr (KS == 2) {
             lds_read16_x4<OFF, OFF, OFF + ARR, OFF + ARR>(opa0, opa1, opa0, opa1, Qf[0], Qf[1], Gf[0], Gf[1]);
@@ -253,21 +304,30 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         } else {
             lds_read16_x4<OFF, OFF + ARR, OFF + ARR, OFF + 2 * ARR>(opa0, opa0, lin, lin, Qf[0], Gf[0], gw[0], ow[0]);
         }
-        // delta[q] = <dO[q], O[q]>: the lanes that share a row sum their pieces (both rows carry
-        // the same permutation of pieces)
+        // the exchanged values: the tiles of the NK key blocks and the rows' sums for delta
+        f32x4 xv[2 * NK + 1];
+        // the lanes that share a row sum their pieces (both rows carry the same permutation of
+        // pieces); afterwards every lane of the row holds the sum over this wavefront's channels
+        xv[2 * NK] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
-            float s = 0.f;
+            float sd = 0.f;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 const uint32_t a = gw[i][w], o = ow[i][w];
-                s = fmaf(to_float<T>((uint16_t)(a & 0xffffu)), to_float<T>((uint16_t)(o & 0xffffu)), s);
-                s = fmaf(to_float<T>((uint16_t)(a >> 16)), to_float<T>((uint16_t)(o >> 16)), s);
+                sd = fmaf(to_float<T>((uint16_t)(a & 0xffffu)), to_float<T>((uint16_t)(o & 0xffffu)), sd);
+                sd = fmaf(to_float<T>((uint16_t)(a >> 16)), to_float<T>((uint16_t)(o >> 16)), sd);
             }
 #pragma unroll
-            for (int m = 1; m < CPR; m <<= 1) s += __shfl_xor(s, m, 64);
-            if (lchk == 0) delta_lds[i * RPI + lrow] = s;
+            for (int m = 1; m < CPR; m <<= 1) sd += __shfl_xor(sd, m, 64);
+            xv[2 * NK][i] = sd;
         }
+#pragma unroll
+        for (int e = 0; e < NK; ++e) leaf_scores(Qf, Gf, Kc[e0 + e], Vc[e0 + e], xv[2 * e], xv[2 * e + 1]);
+        exchange(std::integral_constant<int, 2 * NK + 1>{}, xv);
+#pragma unroll
+        for (int i = 0; i < NLD; ++i)
+            if (lchk == 0) delta_lds[i * RPI + lrow] = xv[2 * NK][i];
         u32x2_t QT[NJ], GT[NJ];
         bt.transpose(Qf, QT);
         bt.transpose(Gf, GT);
@@ -275,7 +335,8 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         const f32x4 dl = *reinterpret_cast<const f32x4 *>(delta_lds + 4 * g);
 #pragma unroll
         for (int i = 0; i < 4; ++i) del4[i] = dl[i];
-        leaf_contrib(Qf, Gf, QT, GT, lse4, del4, Kf, Vf, qb, kb, tk, tv);
+#pragma unroll
+        for (int e = 0; e < NK; ++e) leaf_apply(xv[2 * e], xv[2 * e + 1], QT, GT, lse4, del4, qb, kb0 + e, tk[e], tv[e]);
     };
     auto store_key_block = [&](int kb, const f32x4 (&tk)[NJ], const f32x4 (&tv)[NJ]) {
         bt.put_result(0, tk, 1.0f);
@@ -290,12 +351,11 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     };
 
     // everything the first block needs is requested before anything is consumed
-    u32x4_t Kc[NKB][KS], Vc[NKB][KS];
     u32x4_t rKu[NLD], rVu[NLD];  // the far block's rows on their way
     float halo_lse4[NBW][4];
     using Area0 = std::integral_constant<int, 0>;
-    using Area1 = std::integral_constant<int, STG>;
-    const bool left_halo = !CAUSAL && blk0 > 0, right_halo = blk0 + SB < NB;  // uniform
+    using AreaBefore = std::integral_constant<int, STG>;  // the block before the strip
+    const bool left_halo = !CAUSAL && blk0 > 0;  // uniform
     {
         u32x4_t rKh[NKL][NLD], rVh[NKL][NLD];
         load_far(blk0 * TILE_Q, rKu, rVu);
@@ -308,10 +368,10 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         request_dma(0, blk0);
 #pragma unroll
         for (int c = 0; c + 1 < NKL; ++c) {
-            bt.put(2, rKh[c]);
-            bt.put(3, rVh[c]);
-            bt.get(2, Kc[c]);
-            bt.get(3, Vc[c]);
+            bt.put(0, rKh[c]);
+            bt.put(1, rVh[c]);
+            bt.get(0, Kc[c]);
+            bt.get(1, Vc[c]);
         }
     }
     if constexpr (!CAUSAL) {
@@ -321,7 +381,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) { tk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; tv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
         wait_vmem_all_but<6 * NLD>();  // everything older than the first block's transfers
-        if (left_halo) halo_contrib(Area1{}, halo_lse4[0], blk0 - 1, Kc[1], Vc[1], blk0, tk, tv);
+        if (left_halo) halo_block(AreaBefore{}, std::integral_constant<int, 1>{}, halo_lse4[0], blk0 - 1, 1, blk0, &tk, &tv);
         park_put(0, tk, tv);
     }
     // partial rows of the far block, summed over a run of four blocks
@@ -334,10 +394,10 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         const int q0 = blk * TILE_Q;
         if ((it & (FAR - 1)) == 0) {
             // a new run: its far block (requested a block ahead), nothing summed yet
-            bt.put(2, rKu);
-            bt.put(3, rVu);
-            bt.get(2, Kc[NKL + 1]);
-            bt.get(3, Vc[NKL + 1]);
+            bt.put(0, rKu);
+            bt.put(1, rVu);
+            bt.get(0, Kc[NKL + 1]);
+            bt.get(1, Vc[NKL + 1]);
             far_biases(q0);
             // the strip's second run goes on summing the levels above 6, whose nodes it shares
             // with the first; level 6 (the lanes of slot 0) starts over
@@ -349,28 +409,26 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         u32x4_t Qf[KS], Gf[KS];
         // the next block's rows (after the last block: the neighbour's query block) into the other
         // area, whose reads finished an iteration ago; then everything older is here
-        // The counter the waits look at retires loads, transfers and stores in the order of issue,
-        // so the wait names how many younger operations may still be in flight: the transfers
-        // just requested plus the previous block's stores, which follow this block's request in
-        // program order.  Only stores that are certainly issued are counted (dQ: NLD; the finished
-        // leaf key block: 2 NLD from block NBW of the strip on; near tree rows: 2 NLD, some
-        // lane always has a row); counting too few only waits longer.
+        // This block's rows were requested an iteration ago, right after the block before had
+        // left the area.  The counter the wait looks at retires loads, transfers and stores in the
+        // order of issue, so the wait names how many younger operations may still be in flight:
+        // the previous block's stores, which follow the request in program order.  Only stores
+        // that are certainly issued are counted (dQ: NLD; the finished leaf key block: 2 NLD from
+        // block NBW of the strip on; near tree rows: 2 NLD, some lane always has a row); counting
+        // too few only waits longer.
+        if (it == 0) wait_vmem_all_but<0>();
+        else if (it <= NBW) wait_vmem_all_but<3 * NLD>();
+        else wait_vmem_all_but<5 * NLD>();
+        if constexpr (KS == 2) lds_read16_6x2<0, ARR>(opa0, opa1, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
+        else lds_read16_6x1<0, ARR>(opa0, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
+        // the operands are in registers: the area takes the next block's rows, after the last
+        // block the neighbour's query blocks (three staged blocks each, in the halves of the area)
         if (it + 1 < SB) {
-            request_dma((PAR ^ 1) * STG, blk + 1);
-            if (it == 0) wait_vmem_all_but<6 * NLD>();
-            else if (it <= NBW) wait_vmem_all_but<6 * NLD + 3 * NLD>();
-            else wait_vmem_all_but<6 * NLD + 5 * NLD>();
+            request_dma(0, blk + 1);
         } else {
-            // the neighbour's query blocks, three staged blocks each, into the halves of the area
 #pragma unroll
-            for (int hq = 0; hq < NBW; ++hq) request_halo_dma((PAR ^ 1) * STG + hq * 3 * ARR, blk0 + SB + hq, halo_lse4[hq]);
-            static_assert(SB - 2 >= NBW, "the block before the last stored all of the above");
-            wait_vmem_all_but<NBW * (3 * NLD + 4) + 5 * NLD>();
+            for (int hq = 0; hq < NBW; ++hq) request_halo_dma(hq * 3 * ARR, blk0 + SB + hq, halo_lse4[hq]);
         }
-        if constexpr (KS == 2)
-            lds_read16_6x2<PAR * STG, ARR>(opa0, opa1, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
-        else
-            lds_read16_6x1<PAR * STG, ARR>(opa0, Qf, Gf, Kc[NKL - 1], Vc[NKL - 1], Kc[NKL], Vc[NKL]);
         if constexpr (SB > FAR)
             if ((it & (FAR - 1)) == FAR - 1 && it + 1 < SB) load_far(q0 + TILE_Q, rKu, rVu);  // the next run's far block
 
@@ -416,20 +474,29 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
         // ---- orientation 1: S^T, dP^T [key, query] ---------------------------------------------------
         float sc[NKB][4], dp[NKB][4];
         float mx = NEG_INF;
+        {
+            f32x4 ad[2 * NKB];  // this wavefront's channels' part of the tiles, completed by the exchange
 #pragma unroll
-        for (int c = 0; c < NKB; ++c) {
-            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < NKB; ++c) {
+                f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                a = M_::k32(Kc[c][ks], Qf[ks], a);
-                d = M_::k32(Vc[c][ks], Gf[ks], d);
+                for (int ks = 0; ks < KS; ++ks) {
+                    a = M_::k32(Kc[c][ks], Qf[ks], a);
+                    d = M_::k32(Vc[c][ks], Gf[ks], d);
+                }
+                ad[2 * c] = a;
+                ad[2 * c + 1] = d;
             }
+            exchange(std::integral_constant<int, 2 * NKB>{}, ad);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
-                sc[c][i] = fmaf(a[i], p.scale_log2e, bias);
-                dp[c][i] = d[i];
-                mx = fmaxf(mx, sc[c][i]);
+            for (int c = 0; c < NKB; ++c) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float bias = c < NKL ? biasL[c < NKL ? c : 0][i] : (c == NKL ? b1T[i] : b1U[i]);
+                    sc[c][i] = fmaf(ad[2 * c][i], p.scale_log2e, bias);
+                    dp[c][i] = ad[2 * c + 1][i];
+                    mx = fmaxf(mx, sc[c][i]);
+                }
             }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -474,7 +541,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
                 for (int j = 0; j < NJ; ++j) acc[j] = M_::k16(KT[j], dsp, acc[j]);
             }
             bt.put_result(0, acc, 1.0f);
-            uint16_t *optr = p.dq + ((size_t)b * N * H + h) * D + 8 * lchk + (size_t)(q0 + lrow) * rs;
+            uint16_t *optr = p.dq + qo + 8 * lchk + (size_t)(q0 + lrow) * rs;
 #pragma unroll
             for (int i = 0; i < NLD; ++i)
                 *reinterpret_cast<u32x4_t *>(optr + (size_t)(i * RPI) * rs) = bt.get_row_piece(0, i);
@@ -490,6 +557,12 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             lse4[i] = __shfl(lse, 4 * g + i, 64);
             del4[i] = __shfl(delta, 4 * g + i, 64);
         }
+        // second orientation, S[query 4g+i, key or slot r16] and dP[query, key]: every key block's
+        // tiles first (this wavefront's channels' part, completed by the exchange)
+        f32x4 ad2[2 * NKB];
+#pragma unroll
+        for (int c = 0; c < NKB; ++c) leaf_scores(Qf, Gf, Kc[c], Vc[c], ad2[2 * c], ad2[2 * c + 1]);
+        exchange(std::integral_constant<int, 2 * NKB>{}, ad2);
         // the strip's own leaf key blocks this query block reaches, oldest first: the block before
         // the query block is complete afterwards and leaves; the others wait in registers
 #pragma unroll
@@ -505,7 +578,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
                 } else {
                     park_get(SLOT, tk, tv);
                 }
-                leaf_contrib(Qf, Gf, QT, GT, lse4, del4, Kc[c], Vc[c], blk, blk0 + j, tk, tv);
+                leaf_apply(ad2[2 * c], ad2[2 * c + 1], QT, GT, lse4, del4, blk, blk0 + j, tk, tv);
                 if (c == 0) store_key_block(blk0 + j, tk, tv);
                 else park_put(SLOT, tk, tv);
             }
@@ -513,12 +586,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int c = NKL + t;
-            f32x4 a = {0.f, 0.f, 0.f, 0.f}, d = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                a = M_::k32(Qf[ks], Kc[c][ks], a);   // S[query 4g+i, slot r16]
-                d = M_::k32(Gf[ks], Vc[c][ks], d);   // dP[query, slot]
-            }
+            const f32x4 a = ad2[2 * c], d = ad2[2 * c + 1];  // S[query 4g+i, slot r16], dP[query, slot]
             float pp[4], ds[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -544,12 +612,12 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
                         const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
                         if constexpr (PAR == 1) {
                             const f32x4 ck = *reinterpret_cast<const f32x4 *>(carry + ch);
-                            const f32x4 cv = *reinterpret_cast<const f32x4 *>(carry + D + ch);
+                            const f32x4 cv = *reinterpret_cast<const f32x4 *>(carry + HD + ch);
                             tk[j] += ck;
                             tv[j] += cv;
                         } else {
                             *reinterpret_cast<f32x4 *>(carry + ch) = tk[j];
-                            *reinterpret_cast<f32x4 *>(carry + D + ch) = tv[j];
+                            *reinterpret_cast<f32x4 *>(carry + HD + ch) = tv[j];
                         }
                     }
                 }
@@ -583,8 +651,8 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
                 float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
                 const int run = r16 == 0 ? blk / FAR : blk0 / FAR;
                 const size_t po = ((((size_t)b * NR + run) * H + h) * LF + (lvl - 6)) * D;
-                float *pkp = far + po;
-                float *pvp = far + (size_t)p.B * NR * H * LF * D + po;
+                float *pkp = far + po + half * HD;
+                float *pvp = far + (size_t)p.B * NR * H * LF * D + po + half * HD;
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
                     const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
@@ -621,21 +689,19 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     // NBW - hq of them)
     {
         static_assert(SB % 2 == 0, "the neighbour's blocks are staged in the first area");
+        f32x4 tk[NBW][NJ], tv[NBW][NJ];
+#pragma unroll
+        for (int e = 0; e < NBW; ++e) park_get(((SB - NBW + e) & 1) & (NPARK - 1), tk[e], tv[e]);
         wait_vmem_all_but<0>();
-#pragma unroll
-        for (int e = 0; e < NBW; ++e) {  // key block blk0 + SB - NBW + e, operands in slot e
-            const int j = SB - NBW + e;
-            f32x4 tk[NJ], tv[NJ];
-            park_get((j & 1) & (NPARK - 1), tk, tv);
-#pragma unroll
-            for (int hq = 0; hq <= e; ++hq) {
-                if (blk0 + SB + hq < NB) {  // uniform
-                    if (hq == 0) halo_contrib(Area0{}, halo_lse4[0], blk0 + SB, Kc[e], Vc[e], blk0 + j, tk, tv);
-                    else halo_contrib(std::integral_constant<int, 3 * ARR>{}, halo_lse4[NBW - 1], blk0 + SB + hq, Kc[e], Vc[e], blk0 + j, tk, tv);
-                }
-            }
-            store_key_block(blk0 + j, tk, tv);
+        if (blk0 + SB < NB)  // uniform; the sequence's block count is a multiple of the strip's, so all NBW exist
+            halo_block(Area0{}, std::integral_constant<int, NBW>{}, halo_lse4[0], blk0 + SB, 0, blk0 + SB - NBW, tk, tv);
+        if constexpr (NBW == 2) {
+            if (blk0 + SB < NB)
+                halo_block(std::integral_constant<int, 3 * ARR>{}, std::integral_constant<int, 1>{}, halo_lse4[NBW - 1],
+                           blk0 + SB + 1, 1, blk0 + SB - 1, tk + 1, tv + 1);
         }
+#pragma unroll
+        for (int e = 0; e < NBW; ++e) store_key_block(blk0 + SB - NBW + e, tk[e], tv[e]);
     }
 }
 
@@ -654,31 +720,33 @@ int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t 
 
 // strips of eight blocks where the sequence has that many (one neighbour's block per 128 queries
 // instead of per 64, every wavefront slot of the chip filled once at B8 H8 N2048), else of four
+// launches one variant: a workgroup is four wavefronts (heads), or the two halves of one head
+template <typename T, int D, bool CAUSAL, int SB, int NBW>
+static int bwd_fused_launch_one(const BwdFusedParams &q, hipStream_t st) {
+    constexpr int SPLIT = D > 64 ? 2 : 1;
+    constexpr int WPB = SPLIT == 2 ? 2 : BWD_WPB;
+    const int nwg = SPLIT == 2 ? q.t.n_units : (q.t.n_units + WPB - 1) / WPB;
+    attn_bwd_tile_fused_kernel<T, D, CAUSAL, SB, NBW, SPLIT><<<dim3(nwg), dim3(WPB * 64), 0, st>>>(q);
+    return check_launch("attn_bwd_tile_fused_kernel");
+}
+
 #define HSA_BWD_FUSED_INSTANTIATE(T, D)                                                                     \
     template <>                                                                                             \
     int attn_bwd_fused_launch_td<T, D>(const BwdFusedParams &fp, bool causal, hipStream_t st) {             \
         BwdFusedParams q = fp;                                                                              \
         const int NB = fp.t.N / TILE_Q;                                                                     \
-        const bool fills = (long)(fp.t.n_units / 8) >= 1024; /* one wavefront per SIMD on 256 CUs */       \
+        /* strips of eight where their wavefronts still fill the chip (one per SIMD on 256 CUs) */          \
+        const long waves8 = (long)(fp.t.n_units / 8) * (D > 64 ? 2 : 1);                                    \
         const int knob = bwd_fused_strip_knob();                                                            \
-        const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D == 64 && fills))) ? 8 : 4;             \
+        const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D >= 64 && waves8 >= 1024))) ? 8 : 4;    \
         const int nbw = fp.t.R > TILE_Q ? 2 : 1;                                                            \
         if (nbw == 2 && !causal) return fail(HSA_ERR_UNSUPPORTED, "one-pass backward: window radius above 16 needs the causal mask"); \
         q.t.n_units = fp.t.n_units / sb;                                                                    \
         q.t.red_lg_sb = sb == 8 ? 3 : 2;                                                                    \
-        const int nwg = (q.t.n_units + BWD_WPB - 1) / BWD_WPB;                                              \
-        const dim3 grid(nwg), block(BWD_WPB * 64);                                                          \
-        if (nbw == 2) {                                                                                     \
-            if (sb == 8) attn_bwd_tile_fused_kernel<T, D, true, 8, 2><<<grid, block, 0, st>>>(q);           \
-            else attn_bwd_tile_fused_kernel<T, D, true, 4, 2><<<grid, block, 0, st>>>(q);                   \
-        } else if (sb == 8) {                                                                               \
-            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 8, 1><<<grid, block, 0, st>>>(q);            \
-            else attn_bwd_tile_fused_kernel<T, D, false, 8, 1><<<grid, block, 0, st>>>(q);                  \
-        } else {                                                                                            \
-            if (causal) attn_bwd_tile_fused_kernel<T, D, true, 4, 1><<<grid, block, 0, st>>>(q);            \
-            else attn_bwd_tile_fused_kernel<T, D, false, 4, 1><<<grid, block, 0, st>>>(q);                  \
-        }                                                                                                   \
-        int rc = check_launch("attn_bwd_tile_fused_kernel");                                                \
+        int rc;                                                                                             \
+        if (nbw == 2) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 2>(q, st) : bwd_fused_launch_one<T, D, true, 4, 2>(q, st); \
+        else if (causal) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 1>(q, st) : bwd_fused_launch_one<T, D, true, 4, 1>(q, st); \
+        else rc = sb == 8 ? bwd_fused_launch_one<T, D, false, 8, 1>(q, st) : bwd_fused_launch_one<T, D, false, 4, 1>(q, st); \
         if (rc != HSA_OK || q.t.red_wgs == 0) return rc;                                                    \
         attn_bwd_reduce_kernel<T><<<q.t.red_wgs, BWD_WPB * 64, 0, st>>>(q.t, D);                            \
         return check_launch("attn_bwd_reduce_kernel");                                                      \

@@ -1,0 +1,4 @@
+#include "hsa_attn_bwd_fused.h"
+namespace hsa {
+HSA_BWD_FUSED_INSTANTIATE(BF16, 128)
+}  // namespace hsa

@@ -21,23 +21,20 @@ static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
     return check_launch("attn_tile_kernel");
 }
 
-// the variant that also writes the queries' log-sum-exp (window radius up to 16, up to 64 channels)
+// the variant that also writes the queries' log-sum-exp (window radius up to 16, or 32 with the
+// causal mask)
 template <typename T, int D, int NBW, bool CAUSAL>
 static int tile_launch_lse(const TileParams &p, int sb, int wpb, hipStream_t st) {
-    if constexpr (D <= 64) {
-        constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
-        if (wpb > MAXW) wpb = MAXW;
-        const int nwg = (p.n_units + wpb - 1) / wpb;
-        switch (sb) {
-            case 1: attn_tile_kernel<T, D, NBW, CAUSAL, 1, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
-            case 2: attn_tile_kernel<T, D, NBW, CAUSAL, 2, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
-            case 4: attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
-            default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
-        }
-        return check_launch("attn_tile_kernel (log-sum-exp)");
-    } else {
-        return fail(HSA_ERR_UNSUPPORTED, "the log-sum-exp output is built for up to 64 channels per head");
+    constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
+    if (wpb > MAXW) wpb = MAXW;
+    const int nwg = (p.n_units + wpb - 1) / wpb;
+    switch (sb) {
+        case 1: attn_tile_kernel<T, D, NBW, CAUSAL, 1, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+        case 2: attn_tile_kernel<T, D, NBW, CAUSAL, 2, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+        case 4: attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+        default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
     }
+    return check_launch("attn_tile_kernel (log-sum-exp)");
 }
 
 template <typename T, int D, int NBW, bool CAUSAL>

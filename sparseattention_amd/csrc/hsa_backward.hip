@@ -757,8 +757,11 @@ int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t 
 
 static bool attn_bwd_fused_eligible(int N, int M, int D, int L, int R, int dtype, int causal) {
     if (dtype != HSA_F16 && dtype != HSA_BF16) return false;
-    if (D != 32 && D != 64) return false;
+    if (D != 32 && D != 64 && D != 128) return false;
     if (N < TILE_Q * BWD_STRIP || ilog2_exact(N) != L || L > TILE_MAX_LEVELS || M < 2 * N - 1) return false;
+    // 128 channels (two wavefronts per head) only with the causal mask: without it the exchange
+    // buffers leave room for one workgroup per CU
+    if (D == 128 && causal == 0) return false;
     // one block of neighbours to either side, or two with the causal mask
     return R <= TILE_Q || (R <= 2 * TILE_Q && causal != 0);
 }
@@ -799,7 +802,8 @@ static int attn_bwd_fused_typed(const void *q, const void *k, const void *v, con
     p.red_wgs = (int)red_wgs;
     p.red_lg_sb = 2;
     return D == 32 ? attn_bwd_fused_launch_td<T, 32>(fp, causal != 0, st)
-                   : attn_bwd_fused_launch_td<T, 64>(fp, causal != 0, st);
+         : D == 64 ? attn_bwd_fused_launch_td<T, 64>(fp, causal != 0, st)
+                   : attn_bwd_fused_launch_td<T, 128>(fp, causal != 0, st);
 }
 
 }  // namespace hsa
@@ -942,7 +946,7 @@ int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *
     HSA_REQUIRE(R >= 0, "bad R=%d", R);
     if (!hsa::attn_bwd_fused_eligible(N, M, D, L, R, dtype, causal))
         return hsa::fail(HSA_ERR_UNSUPPORTED, "one-pass backward not available for N=%d D=%d L=%d R=%d causal=%d dtype=%d "
-                         "(16-bit types, 32 or 64 channels per head, radius up to 16, or up to 32 with the causal mask, "
+                         "(16-bit types, 32, 64 or 128 channels per head, radius up to 16, or up to 32 with the causal mask, "
                          "at least 64 leaves)", N, D, L, R, causal ? 1 : 0, dtype);
     const bool aligned = (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out | (uintptr_t)dout |
                            (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv | (uintptr_t)workspace) & 15) == 0;

@@ -26,6 +26,14 @@ namespace hsa {
 // LDS byte address of a pointer into a __shared__ array (the low half of its flat address)
 __device__ __forceinline__ uint32_t lds_address(const void *p) { return (uint32_t)(uintptr_t)p; }
 
+// workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for every
+// vector-memory operation in flight, the transfers requested ahead included
+__device__ __forceinline__ void lds_only_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // one instruction: lane l's 16 bytes from g to LDS[lds_base + 16 l]; lds_base is wavefront-uniform
 __device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds_base) {
     uint32_t keep;

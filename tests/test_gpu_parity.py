@@ -1075,7 +1075,9 @@ def test_attention_backward_wide_window_128_channels_both_formulations(dtype, ca
 SAVED_BWD_CASES = [(2, 64, 2, 64, 16), (1, 128, 3, 64, 5), (2, 256, 4, 32, 16), (1, 512, 2, 64, 0), (2, 1024, 8, 64, 16),
                    (1, 2048, 2, 32, 9), (3, 64, 1, 32, 1), (1, 128, 1, 32, 16), (1, 4096, 3, 64, 13),
                    # window radius 17..32: two blocks of neighbours, with the causal mask only
-                   (2, 64, 2, 64, 32), (1, 128, 3, 64, 17), (2, 256, 2, 32, 32), (1, 1024, 4, 64, 25), (1, 2048, 1, 32, 20)]
+                   (2, 64, 2, 64, 32), (1, 128, 3, 64, 17), (2, 256, 2, 32, 32), (1, 1024, 4, 64, 25), (1, 2048, 1, 32, 20),
+                   # 128 channels per head: two wavefronts per head, with the causal mask only
+                   (1, 64, 2, 128, 16), (2, 128, 1, 128, 32), (1, 512, 2, 128, 9), (1, 1024, 3, 128, 32), (2, 256, 2, 128, 20)]
 
 
 @pytest.mark.parametrize("case", SAVED_BWD_CASES)
@@ -1088,7 +1090,7 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
     log-sum-exp against the oracle's logits.  One strip (no neighbours), first / last strips and
     inner strips all occur."""
     B, N, H, D, R = case
-    if R > 16 and not causal:
+    if (R > 16 or D == 128) and not causal:
         qz = torch.zeros(B, N, H, D, dtype=dtype, device=DEV)
         assert not fn.saved_state_backward_available(qz, torch.zeros(B, 2 * N - 1, H, D, dtype=dtype, device=DEV), R, False)
         return
@@ -1161,8 +1163,11 @@ def test_attention_backward_saved_state_limits():
     assert fn.saved_state_backward_available(q, k, 32, True) and not fn.saved_state_backward_available(q, k, 33, True)
     assert not fn.saved_state_backward_available(q.float(), k.float(), 16)      # fp32
     assert not fn.saved_state_backward_available(q[:, :32], k[:, :63], 16)      # fewer than 64 leaves
-    q128 = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16, device=DEV)
-    assert not fn.saved_state_backward_available(q128, torch.zeros(1, 127, 2, 128, dtype=torch.bfloat16, device=DEV), 16)
+    q128, k128 = (torch.zeros(1, rows, 2, 128, dtype=torch.bfloat16, device=DEV) for rows in (64, 127))
+    assert fn.saved_state_backward_available(q128, k128, 16, True)
+    assert not fn.saved_state_backward_available(q128, k128, 16, False)         # 128 channels without the mask
+    q256, k256 = (torch.zeros(1, rows, 2, 256, dtype=torch.bfloat16, device=DEV) for rows in (64, 127))
+    assert not fn.saved_state_backward_available(q256, k256, 16, True)
     lib = _lib.lib()
     d = _lib.ptr(q)
     rc = lib.hsa_attn_bwd_saved(d, d, d, d, d, d, d, d, d, d, 1 << 20, 1, 64, 127, 2, 64, 6, 17, 0, 2, _lib.stream_of(q))
