@@ -417,8 +417,9 @@ class BuildParentNodesFunc(torch.autograd.Function):
 
 # Which backward `hierarchical_attention` uses.  Two formulations exist: two passes over Q, dO and
 # the leaf K / V (any shape the tile kernels take), and one pass that works from the forward's
-# output and one log-sum-exp per (query, head), which the forward then keeps (16-bit types, 32 / 64
-# channels per head, window radius up to 16).  The one pass moves less (0.76 of the two passes' HBM
+# output and one log-sum-exp per (query, head), which the forward then keeps (16-bit types; 32 / 64
+# channels per head with window radius up to 16, or up to 32 with the causal mask; 128 channels
+# with the causal mask).  The one pass moves less (0.76 of the two passes' HBM
 # traffic at B8 H8 N2048 D64) and measured faster on every shape tried (50.8 against 56.4 us there,
 # 29.6 against 34.7 us at B16 H8 N512, 64.0 against 68.9 us at B2 H16 N8192 D32, 53.8 against 58.7 us
 # at B8 H8 N2048 without the causal mask).
