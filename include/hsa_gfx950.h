@@ -174,9 +174,13 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
  * unless `out` allows the launch per level, which takes any power of two.
  * hsa_cross_update_level_rows returns the C from which on a caller with such an `out` should hand
  * the remaining levels to hsa_cross_update_top_fwd instead of running a GEMM and a parent build
- * per level: at least hsa_cross_update_top_rows, more for small batches (B*C <= 4096).
+ * per level: at least hsa_cross_update_top_rows, more for small batches (B*C <= 8192).
+ * hsa_cross_update_level_tune (experiments and tests; -1 keeps a value): levels with at least
+ * wg_min_tiles 16-row tiles run on the kernel that stages a head's weights in LDS once per
+ * workgroup (0: never), and rows_limit replaces the 8192 above.  Process-wide.
  */
 int hsa_cross_update_top_tune(int single_launch);
+int hsa_cross_update_level_tune(int wg_min_tiles, long rows_limit);
 int hsa_cross_update_top_rows(int H, int Dh, int dtype);
 int hsa_cross_update_level_rows(int B, int H, int Dh, int dtype);
 int hsa_cross_update_pack_weights(const void *wk, const void *wv, void *packed, int H, int Dh,

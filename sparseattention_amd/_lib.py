@@ -34,6 +34,8 @@ def _declare(lib):
     lib.hsa_attn_fwd.restype = I
     lib.hsa_attn_fwd_timed.argtypes = [P, P, P, P, P, P, P] + [I] * 10 + [P, P, P]
     lib.hsa_attn_fwd_timed.restype = I
+    lib.hsa_cross_update_level_tune.argtypes = [I, ctypes.c_long]
+    lib.hsa_cross_update_level_tune.restype = I
     lib.hsa_attn_bwd_tables.argtypes = [P] * 11 + [ctypes.c_size_t] + [I] * 9 + [P]
     lib.hsa_attn_bwd_tables.restype = I
     lib.hsa_attn_bwd_saved_tune.argtypes = [I]

@@ -16,6 +16,7 @@
 // lanes that share those rows.  The level's output goes to the result tensor and to the other
 // LDS buffer, which is the next level's input.
 #include "hsa_mma.h"
+#include "hsa_lds_dma.h"
 
 #include <stdlib.h>
 
@@ -239,6 +240,180 @@ __global__ void __launch_bounds__(64) cross_update_level_kernel(TopParams p, int
                                           lsrc_rs * 2, RT * (int)blockIdx.z);
 }
 
+
+// One level per launch for the LARGE levels: a workgroup of WAVES wavefronts shares one (batch
+// element, head) and WAVES * RT row tiles of 16 children.  The head's key and value projection
+// weights are staged in LDS once per workgroup (chunks of KC k-steps, both halves, two buffers:
+// the next chunk is transferred global -> LDS without a stop in the registers while the current
+// one is multiplied), so they are fetched once per WAVES * RT * 16 rows instead of once per
+// wavefront, and both projections run in one pass over the children's rows (accumulators of both
+// halves live side by side), so those rows are read once.  In the packed order a lane's operand of
+// (half, k-step, column tile) is 16 consecutive bytes and a wavefront's 1 KiB: the transfer puts
+// it at 16 * lane, which is also a conflict-free read.  The 3-way softmax and the weighted sum
+// finish from the accumulators exactly like top_level_head (same rounding points), so the level
+// needs no projection GEMM, no [rows, 2 Dm] intermediate and no separate parent build.
+// OCC = workgroups per CU the kernel is compiled for (2: at most 256 registers; the weights'
+// operands are then read a k-step at a time, the other workgroup covers the wait)
+template <typename T, int CT2, int RT, int WAVES, int KC, int OCC = 1>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(OCC)))
+cross_update_level_wg_kernel(TopParams p, int C, int row,
+                                                                           const uint16_t *lsrc, int64_t lsrc_bs,
+                                                                           int64_t lsrc_rs) {
+#pragma clang fp contract(off)
+    using M_ = Mma<T>;
+    extern __shared__ __align__(16) unsigned char wlds[];
+    constexpr int Dh = 16 * CT2;
+    constexpr int CHB = 2 * KC * CT2 * 1024;     // one buffer: [half][k-step][column tile][lane][16 bytes]
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+    const int Dm = p.Dm, NK = Dm / 32, NCH = NK / KC, P = C >> 1;
+    const int tile0 = ((int)blockIdx.z * WAVES + wave) * RT;
+    const unsigned char *cur = reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs);
+    const int64_t pitch = lsrc_rs * 2;
+    const unsigned char *arow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int r = 16 * (tile0 + rt) + r16;
+        arow[rt] = cur + (int64_t)(r < C ? r : C - 1) * pitch + 16 * g;
+    }
+    // parent e of row tile rt in this lane: 8(tile0 + rt) + 2g + e, children = accumulator rows 2e, 2e+1
+    const uint16_t *prow[RT][2];
+    bool valid[RT][2];
+    int prel[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int pe = 8 * (tile0 + rt) + 2 * g + e;
+            valid[rt][e] = pe < P;
+            prel[rt][e] = valid[rt][e] ? pe : P - 1;
+            prow[rt][e] = p.qkv + (size_t)b * p.qkv_bs + (size_t)(row + prel[rt][e]) * p.qkv_rs + h * Dh + r16;
+        }
+
+    // the head's packed weights: [half][head][k-step][column tile][lane][8 elements]
+    const uint16_t *wsrc[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) wsrc[half] = p.w + ((size_t)(half * p.H + h) * NK * CT2 * 64 + lane) * 8;
+    const uint32_t lbase = lds_address(wlds);
+    // chunk c -> buffer c & 1: 2 * KC * CT2 pieces of 1 KiB, dealt to the wavefronts in turn
+    auto issue = [&](int c) {
+        const uint32_t dst = lbase + (c & 1) * CHB;
+        for (int i = wave; i < 2 * KC * CT2; i += WAVES) {
+            const int half = i / (KC * CT2), j = i - half * (KC * CT2);
+            lds_dma16(wsrc[half] + (size_t)(c * KC * CT2 + j) * 512, dst + i * 1024);
+        }
+    };
+
+    f32x4 accK[RT][CT2], accV[RT][CT2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT2; ++ct) {
+            accK[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+            accV[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    // The children's rows of a whole chunk are requested a chunk ahead (a ring of KC k-steps in
+    // registers), the weights' operands of a k-step one k-step ahead (from LDS): with one
+    // wavefront per SIMD nothing else hides those latencies.
+    u32x4_t aq[KC][RT];
+    auto load_a = [&](int u, int kg) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) aq[u][rt] = *reinterpret_cast<const u32x4_t *>(arow[rt] + 64 * kg);
+    };
+    auto load_b = [&](u32x4_t (&bq)[2 * CT2], const unsigned char *wb, int ks) {
+#pragma unroll
+        for (int ct = 0; ct < CT2; ++ct) {
+            bq[ct] = *reinterpret_cast<const u32x4_t *>(wb + ((0 * KC + ks) * CT2 + ct) * 1024);
+            bq[CT2 + ct] = *reinterpret_cast<const u32x4_t *>(wb + ((1 * KC + ks) * CT2 + ct) * 1024);
+        }
+    };
+    // the parents' own q, k, v (needed after the projection) are requested first: they arrive
+    // behind the main loop
+    uint16_t rq[RT][2][CT2], rk[RT][2][CT2], rv[RT][2][CT2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+            for (int c = 0; c < CT2; ++c) {
+                rq[rt][e][c] = prow[rt][e][16 * c];
+                rk[rt][e][c] = prow[rt][e][Dm + 16 * c];
+                rv[rt][e][c] = prow[rt][e][2 * Dm + 16 * c];
+            }
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+    issue(0);
+#pragma unroll
+    for (int u = 0; u < KC; ++u) load_a(u, u);  // NK >= KC
+    __builtin_amdgcn_sched_barrier(0);
+
+    for (int c = 0; c < NCH; ++c) {
+        // this chunk's transfers (requested a chunk ago) are complete in every wavefront, and
+        // every wavefront has finished reading the buffer the next chunk goes to
+        // (younger than those transfers: the KC * RT row loads issued since, which stay in flight)
+        asm volatile("" ::: "memory");
+        wait_vmem_all_but<KC * RT>();
+        lds_only_barrier();
+        const bool more = c + 1 < NCH;
+        if (more) issue(c + 1);
+        const unsigned char *wb = wlds + (c & 1) * CHB + lane * 16;
+        constexpr int NBQ = OCC >= 2 ? 1 : 2;
+        u32x4_t bq[NBQ][2 * CT2];
+        if constexpr (NBQ == 2) load_b(bq[0], wb, 0);
+#pragma unroll
+        for (int ks = 0; ks < KC; ++ks) {
+            u32x4_t a[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) a[rt] = aq[ks][rt];
+            if (more) load_a(ks, (c + 1) * KC + ks);
+            if constexpr (NBQ == 2) {
+                if (ks + 1 < KC) load_b(bq[(ks + 1) & 1], wb, ks + 1);
+            } else {
+                load_b(bq[0], wb, ks);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ct = 0; ct < CT2; ++ct)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    accK[rt][ct] = M_::k32(a[rt], bq[ks & (NBQ - 1)][ct], accK[rt][ct]);
+                    accV[rt][ct] = M_::k32(a[rt], bq[ks & (NBQ - 1)][CT2 + ct], accV[rt][ct]);
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- the three scores and the softmax weights, then the weighted sum of the values ----
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+            for (int c = 0; c < CT2; ++c) {
+                const float fq = to_float<T>(rq[rt][e][c]);
+                s0 = fmaf(fq, to_float<T>(rk[rt][e][c]), s0);
+                s1 = fmaf(fq, rounded<T>(accK[rt][c][2 * e]), s1);
+                s2 = fmaf(fq, rounded<T>(accK[rt][c][2 * e + 1]), s2);
+            }
+            s0 = group_sum(s0, 16);
+            s1 = group_sum(s1, 16);
+            s2 = group_sum(s2, 16);
+            float w0, w1, w2;
+            softmax3<T>(s0 * p.scale, s1 * p.scale, s2 * p.scale, w0, w1, w2);
+            uint16_t *orow = p.out + (size_t)b * p.out_bs + (size_t)(row + prel[rt][e]) * p.out_rs + h * Dh + r16;
+#pragma unroll
+            for (int c = 0; c < CT2; ++c) {
+                // explicit fused multiply-adds: every variant of the level rounds at the same places
+                const float o = fmaf(w2, rounded<T>(accV[rt][c][2 * e + 1]),
+                                     fmaf(w1, rounded<T>(accV[rt][c][2 * e]), w0 * to_float<T>(rv[rt][e][c])));
+                if (valid[rt][e]) orow[16 * c] = from_float<T>(o);
+            }
+        }
+    }
+}
+
 template <typename T, int CT2, int RT0>
 __global__ void __launch_bounds__(TOP_WAVES * 64) cross_update_top_kernel(TopParams p) {
     extern __shared__ __align__(16) unsigned char top_smem[];
@@ -355,13 +530,82 @@ static bool top_levels_eligible(const TopParams &p) {
            ((uintptr_t)p.src & 15) == 0 && p.src_bs % 8 == 0 && p.Dm % 8 == 0;
 }
 
+// knob for experiments: levels with at least this many 16-row tiles take the workgroup kernel
+// (0: never)
+static std::atomic<int> &level_wg_min_tiles() {
+    static std::atomic<int> v{[] { const char *e = getenv("HSA_CROSS_WG_MIN_TILES"); return e ? atoi(e) : 8; }()};
+    return v;
+}
+
+// batch size times children of the largest level the per-level launches take over from the GEMMs
+static std::atomic<long> &level_rows_limit() {
+    static std::atomic<long> v{[] { const char *e = getenv("HSA_CROSS_LEVEL_ROWS_LIMIT"); return e ? atol(e) : 8192L; }()};
+    return v;
+}
+
+constexpr int LEVEL_WG_WAVES = 4;
+
+template <typename T, int CT2, int RT, int KC, int OCC = 1>
+int launch_level_wg(const TopParams &p, int C, int row, const uint16_t *lsrc, int64_t lbs, int64_t lrs, hipStream_t st) {
+    const size_t lds = 2 * (size_t)(2 * KC * CT2 * 1024);
+    auto kern = cross_update_level_wg_kernel<T, CT2, RT, LEVEL_WG_WAVES, KC, OCC>;
+    if (lds > 64 * 1024) {
+        // raising the limit is slow: once per kernel and device
+        static std::atomic<bool> allowed[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(HSA_ERR_LAUNCH, "no current device");
+        if (!allowed[dev].load(std::memory_order_acquire)) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "LDS size %zu refused: %s", lds, hipGetErrorString(e));
+            allowed[dev].store(true, std::memory_order_release);
+        }
+    }
+    const int tiles = (C + 15) / 16;
+    const dim3 grid((unsigned)p.B, (unsigned)p.H, (unsigned)((tiles + LEVEL_WG_WAVES * RT - 1) / (LEVEL_WG_WAVES * RT)));
+    kern<<<grid, LEVEL_WG_WAVES * 64, lds, st>>>(p, C, row, lsrc, lbs, lrs);
+    return HSA_OK;
+}
+
+// Which variant: two row tiles per wavefront where that still starts a workgroup per CU (else
+// one); two workgroups per CU (chunks of four k-steps: 64 KB of LDS) where there are at least two
+// per CU to start.  Measured at B8 H8 Dh64 (us per level of 4096 / 2048 / 1024 / 512 / 256 / 128
+// children): 68 / 34 / 18.5 / 10.9 / 7.2 / 6.7; a GEMM plus the parent build take 71 / 36 / 26,
+// the launch per wavefront and row tile 18 / 10.4 / 7.2 from 512 children down.
+template <typename T, int CT2>
+int launch_level_wg_any(const TopParams &p, int C, int row, const uint16_t *lsrc, int64_t lbs, int64_t lrs, hipStream_t st) {
+    const int NK = p.Dm / 32;
+    const long tiles = (C + 15) / 16, bh = (long)p.B * p.H;
+    auto wgs = [&](int rt) { return bh * ((tiles + LEVEL_WG_WAVES * rt - 1) / (LEVEL_WG_WAVES * rt)); };
+    if constexpr (CT2 <= 4) {
+        if (wgs(2) >= 512) return launch_level_wg<T, CT2, 2, 4, 2>(p, C, row, lsrc, lbs, lrs, st);
+        if (NK % 8 == 0) {
+            if (wgs(2) >= 256) return launch_level_wg<T, CT2, 2, 8>(p, C, row, lsrc, lbs, lrs, st);
+            return launch_level_wg<T, CT2, 1, 8>(p, C, row, lsrc, lbs, lrs, st);
+        }
+    }
+    if (wgs(2) >= 256) return launch_level_wg<T, CT2, 2, 4>(p, C, row, lsrc, lbs, lrs, st);  // Dm is a multiple of 128
+    return launch_level_wg<T, CT2, 1, 4>(p, C, row, lsrc, lbs, lrs, st);
+}
+
 template <typename T, int CT2, int PD>
 int top_launch_levels_pd(const TopParams &p, hipStream_t st) {
     int C = p.C0, row = 0;
     const uint16_t *lsrc = p.src;
     int64_t lbs = p.src_bs, lrs = p.Dm;
+    const int wg_min = level_wg_min_tiles().load();
     while (C >= 2) {
         const int tiles = (C + 15) / 16;
+        if (wg_min > 0 && tiles >= wg_min) {
+            const int rc = launch_level_wg_any<T, CT2>(p, C, row, lsrc, lbs, lrs, st);
+            if (rc != HSA_OK) return rc;
+            lsrc = p.out + (size_t)row * p.out_rs;
+            lbs = p.out_bs;
+            lrs = p.out_rs;
+            row += C >> 1;
+            C >>= 1;
+            continue;
+        }
         // two row tiles per wavefront where single tiles would need a second round of wavefronts
         // (1024 SIMDs; a lone wavefront's registers hold two tiles' operands up to 64 channels)
         if (CT2 <= 4 && tiles % 2 == 0 && (long)p.B * p.H * tiles >= 2048) {
@@ -422,6 +666,13 @@ int hsa_cross_update_top_tune(int single_launch) {
     return HSA_OK;
 }
 
+int hsa_cross_update_level_tune(int wg_min_tiles, long rows_limit) {
+    if (wg_min_tiles < -1 || rows_limit < -1) return hsa::fail(HSA_ERR_INVALID, "negative knob");
+    if (wg_min_tiles >= 0) hsa::level_wg_min_tiles().store(wg_min_tiles);
+    if (rows_limit >= 0) hsa::level_rows_limit().store(rows_limit);
+    return HSA_OK;
+}
+
 int hsa_cross_update_top_rows(int H, int Dh, int dtype) {
     if (!hsa::top_shape_ok(H, Dh, dtype)) return 0;
     return 16 * hsa::top_row_tiles(H, Dh);
@@ -435,7 +686,8 @@ int hsa_cross_update_level_rows(int B, int H, int Dh, int dtype) {
     // parent build per level while the batch's rows of a level are few (measured on the LM forward
     // at 4096 tokens: up to 4096 rows at batch 1, 1024 at 4, 512 at 8, no gain from 32 on)
     int rows = held;
-    while ((long)B * rows * 2 <= 4096) rows *= 2;
+    const long limit = hsa::level_rows_limit().load();
+    while ((long)B * rows * 2 <= limit) rows *= 2;
     return rows;
 }
 

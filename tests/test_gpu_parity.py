@@ -370,10 +370,45 @@ def test_cross_update_top_many_rows_per_level_launches(B, C, H, Dh, top_knob):
     lib = _lib.lib()
     assert lib.hsa_cross_update_level_rows(B, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
     top_knob(0)
-    assert lib.hsa_cross_update_level_rows(1, H, Dh, _lib.HSA_BF16) == 4096
-    assert lib.hsa_cross_update_level_rows(8, H, Dh, _lib.HSA_BF16) == 512
+    assert lib.hsa_cross_update_level_rows(1, H, Dh, _lib.HSA_BF16) == 8192
+    assert lib.hsa_cross_update_level_rows(8, H, Dh, _lib.HSA_BF16) == 1024
     assert lib.hsa_cross_update_level_rows(4096, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
     assert lib.hsa_cross_update_level_rows(1, 3, 24, _lib.HSA_BF16) == 0
+
+
+@pytest.mark.parametrize("B,C,H,Dh", [(8, 1024, 8, 64), (8, 512, 8, 64), (2, 1024, 8, 64), (16, 256, 4, 32), (4, 512, 2, 128),
+                                      (8, 256, 6, 64), (3, 128, 4, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cross_update_levels_weights_staged_per_workgroup(B, C, H, Dh, dtype):
+    """Large levels run on the kernel that stages a head's weights in LDS once per workgroup (two
+    row tiles per wavefront or one, one or two workgroups per CU, chunks of four or eight k-steps,
+    a model width that is no multiple of 256): bit-identical to the launch per wavefront and row
+    tile, which rounds at the same places, and close to the level-by-level kernels."""
+    dim = H * Dh
+    g = torch.Generator().manual_seed(C + H + B)
+    src = torch.randn(B, C, dim, generator=g).clamp(-1, 1).to(dtype).to(DEV)
+    qkv = torch.randn(B, C - 1, 3 * dim, generator=g).clamp(-1, 1).to(dtype).to(DEV)
+    w = (torch.randn(2 * dim, dim, generator=g) / dim ** 0.5).to(dtype).to(DEV)
+    wp = fn.pack_kv_weights(w[:dim], w[dim:], H)
+    lib = _lib.lib()
+    outs = {}
+    try:
+        for min_tiles in (0, 1):   # never / every level with at least one 16-row tile
+            assert lib.hsa_cross_update_level_tune(min_tiles, -1) == 0
+            outs[min_tiles] = fn.cross_update_top(src, qkv, wp, torch.empty(B, C - 1, dim, dtype=dtype, device=DEV), H)
+    finally:
+        assert lib.hsa_cross_update_level_tune(8, -1) == 0
+    assert torch.equal(outs[0], outs[1])
+    cur, off, P, ref = src, 0, C // 2, []
+    while P >= 1:
+        kv = torch.nn.functional.linear(cur, w).view(B, 2 * P, 2, H, Dh)
+        par = qkv[:, off:off + P].view(B, P, 3, H, Dh)
+        o = torch.empty(B, P, H, Dh, dtype=dtype, device=DEV)
+        fn.build_parents_strided(par[:, :, 0], par[:, :, 1], par[:, :, 2], kv[:, :, 0], kv[:, :, 1], out=o)
+        cur = o.view(B, P, dim)
+        ref.append(cur)
+        off, P = off + P, P // 2
+    assert (outs[1].float() - torch.cat(ref, dim=1).float()).abs().max() < 2e-2
 
 
 def test_cross_update_top_shapes_not_handled(top_knob):
