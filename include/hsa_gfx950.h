@@ -174,10 +174,11 @@ int hsa_build_parents_strided_fwd(const void *qp, const void *kp, const void *vp
  * unless `out` allows the launch per level, which takes any power of two.
  * hsa_cross_update_level_rows returns the C from which on a caller with such an `out` should hand
  * the remaining levels to hsa_cross_update_top_fwd instead of running a GEMM and a parent build
- * per level: at least hsa_cross_update_top_rows, more for small batches (B*C <= 8192).
+ * per level: every level where a head's key and value weights fit 128 KiB of LDS (heads of up to
+ * 64 channels), else at least hsa_cross_update_top_rows and more for small batches (B*C <= 8192).
  * hsa_cross_update_level_tune (experiments and tests; -1 keeps a value): levels with at least
- * wg_min_tiles 16-row tiles run on the kernel that stages a head's weights in LDS once per
- * workgroup (0: never), and rows_limit replaces the 8192 above.  Process-wide.
+ * wg_min_tiles 16-row tiles run on the kernels that keep a head's weights in LDS (0: never), and
+ * rows_limit, when positive, is the bound on B*C for every shape (0: the rule above).  Process-wide.
  */
 int hsa_cross_update_top_tune(int single_launch);
 int hsa_cross_update_level_tune(int wg_min_tiles, long rows_limit);

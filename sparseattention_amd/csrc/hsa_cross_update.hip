@@ -414,6 +414,158 @@ cross_update_level_wg_kernel(TopParams p, int C, int row,
     }
 }
 
+// The LARGEST levels: the same fused level, with the head's whole key and value weights resident
+// in LDS (2 * Dm/32 * Dh/16 KiB: 128 KiB at Dm 512, Dh 64) while a workgroup of eight wavefronts
+// (two per SIMD: one's epilogue runs under the other's multiplications) walks several groups of
+// 16 row tiles.  The weights are transferred once per workgroup and there is no barrier after the
+// first; the children's rows travel through a ring of PD k-steps in registers that runs across
+// the groups, so only a workgroup's very first rows are waited for.
+template <typename T, int CT2, int PD>
+__global__ void __launch_bounds__(512) cross_update_level_pw_kernel(TopParams p, int C, int row, const uint16_t *lsrc,
+                                                                    int64_t lsrc_bs, int64_t lsrc_rs) {
+#pragma clang fp contract(off)
+    using M_ = Mma<T>;
+    extern __shared__ __align__(16) unsigned char wlds[];
+    constexpr int Dh = 16 * CT2, RT = 2, WAVES = 8;
+    const int b = blockIdx.x, h = blockIdx.y, part = blockIdx.z, parts = gridDim.z;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, r16 = lane & 15, g = lane >> 4;
+    const int Dm = p.Dm, NK = Dm / 32, P = C >> 1;
+    const int tiles = (C + 15) / 16, groups = (tiles + WAVES * RT - 1) / (WAVES * RT);
+    const int mine = part < groups ? (groups - part + parts - 1) / parts : 0;  // this workgroup's groups
+    const unsigned char *cur = reinterpret_cast<const unsigned char *>(lsrc + (size_t)b * lsrc_bs);
+    const int64_t pitch = lsrc_rs * 2;
+
+    // the head's packed weights, [half][k-step][column tile][lane][16 bytes], dealt to the wavefronts
+    {
+        const uint32_t lbase = lds_address(wlds);
+        for (int i = wave; i < 2 * NK * CT2; i += WAVES) {
+            const int half = i / (NK * CT2), j = i - half * (NK * CT2);
+            lds_dma16(p.w + ((size_t)(half * p.H + h) * NK * CT2 * 64 + (size_t)j * 64 + lane) * 8, lbase + i * 1024);
+        }
+    }
+    auto rows_of = [&](int gi, const unsigned char *(&ar)[RT]) {  // group gi of this workgroup
+        const int tile0 = ((part + gi * parts) * WAVES + wave) * RT;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const int r = 16 * (tile0 + rt) + r16;
+            ar[rt] = cur + (int64_t)(r < C ? r : C - 1) * pitch + 16 * g;
+        }
+        return tile0;
+    };
+    const unsigned char *arow[RT], *anext[RT];
+    u32x4_t aq[PD][RT];
+    if (mine > 0) {
+        rows_of(0, arow);
+#pragma unroll
+        for (int u = 0; u < PD; ++u)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) aq[u][rt] = *reinterpret_cast<const u32x4_t *>(arow[rt] + 64 * u);  // NK >= PD
+    }
+    asm volatile("" ::: "memory");
+    // the transfers are older than the PD * RT row loads just issued (none if this workgroup has no group)
+    if (mine > 0) wait_vmem_all_but<PD * RT>();
+    else wait_vmem_all_but<0>();
+    lds_only_barrier();
+    const unsigned char *wb = wlds + lane * 16;
+
+    for (int gi = 0; gi < mine; ++gi) {
+        const int tile0 = rows_of(gi, arow);
+        const bool has_next = gi + 1 < mine;
+        if (has_next) rows_of(gi + 1, anext);
+        // parent e of row tile rt in this lane: 8(tile0 + rt) + 2g + e, children = accumulator rows 2e, 2e+1
+        const uint16_t *prow[RT][2];
+        bool valid[RT][2];
+        int prel[RT][2];
+        uint16_t rq[RT][2][CT2], rk[RT][2][CT2], rv[RT][2][CT2];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int pe = 8 * (tile0 + rt) + 2 * g + e;
+                valid[rt][e] = pe < P;
+                prel[rt][e] = valid[rt][e] ? pe : P - 1;
+                prow[rt][e] = p.qkv + (size_t)b * p.qkv_bs + (size_t)(row + prel[rt][e]) * p.qkv_rs + h * Dh + r16;
+#pragma unroll
+                for (int c = 0; c < CT2; ++c) {  // needed after the projection: they arrive behind it
+                    rq[rt][e][c] = prow[rt][e][16 * c];
+                    rk[rt][e][c] = prow[rt][e][Dm + 16 * c];
+                    rv[rt][e][c] = prow[rt][e][2 * Dm + 16 * c];
+                }
+            }
+        f32x4 accK[RT][CT2], accV[RT][CT2];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int ct = 0; ct < CT2; ++ct) {
+                accK[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+                accV[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        for (int ks0 = 0; ks0 < NK; ks0 += PD) {
+#pragma unroll
+            for (int u = 0; u < PD; ++u) {
+                const int ks = ks0 + u;
+                u32x4_t a[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) a[rt] = aq[u][rt];
+                // the ring runs on into the next group's rows
+                const int kn = ks + PD;
+                if (kn < NK) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) aq[u][rt] = *reinterpret_cast<const u32x4_t *>(arow[rt] + 64 * kn);
+                } else if (has_next) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) aq[u][rt] = *reinterpret_cast<const u32x4_t *>(anext[rt] + 64 * (kn - NK));
+                }
+                u32x4_t bq[2 * CT2];
+#pragma unroll
+                for (int ct = 0; ct < CT2; ++ct) {
+                    bq[ct] = *reinterpret_cast<const u32x4_t *>(wb + ((size_t)(0 * NK + ks) * CT2 + ct) * 1024);
+                    bq[CT2 + ct] = *reinterpret_cast<const u32x4_t *>(wb + ((size_t)(1 * NK + ks) * CT2 + ct) * 1024);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int ct = 0; ct < CT2; ++ct)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        accK[rt][ct] = M_::k32(a[rt], bq[ct], accK[rt][ct]);
+                        accV[rt][ct] = M_::k32(a[rt], bq[CT2 + ct], accV[rt][ct]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // ---- the three scores and the softmax weights, then the weighted sum of the values ----
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int c = 0; c < CT2; ++c) {
+                    const float fq = to_float<T>(rq[rt][e][c]);
+                    s0 = fmaf(fq, to_float<T>(rk[rt][e][c]), s0);
+                    s1 = fmaf(fq, rounded<T>(accK[rt][c][2 * e]), s1);
+                    s2 = fmaf(fq, rounded<T>(accK[rt][c][2 * e + 1]), s2);
+                }
+                s0 = group_sum(s0, 16);
+                s1 = group_sum(s1, 16);
+                s2 = group_sum(s2, 16);
+                float w0, w1, w2;
+                softmax3<T>(s0 * p.scale, s1 * p.scale, s2 * p.scale, w0, w1, w2);
+                uint16_t *orow = p.out + (size_t)b * p.out_bs + (size_t)(row + prel[rt][e]) * p.out_rs + h * Dh + r16;
+#pragma unroll
+                for (int c = 0; c < CT2; ++c) {
+                    // explicit fused multiply-adds: every variant of the level rounds at the same places
+                    const float o = fmaf(w2, rounded<T>(accV[rt][c][2 * e + 1]),
+                                         fmaf(w1, rounded<T>(accV[rt][c][2 * e]), w0 * to_float<T>(rv[rt][e][c])));
+                    if (valid[rt][e]) orow[16 * c] = from_float<T>(o);
+                }
+            }
+        }
+    }
+}
+
 template <typename T, int CT2, int RT0>
 __global__ void __launch_bounds__(TOP_WAVES * 64) cross_update_top_kernel(TopParams p) {
     extern __shared__ __align__(16) unsigned char top_smem[];
@@ -538,9 +690,16 @@ static std::atomic<int> &level_wg_min_tiles() {
 }
 
 // batch size times children of the largest level the per-level launches take over from the GEMMs
+// (0: chosen by shape)
 static std::atomic<long> &level_rows_limit() {
-    static std::atomic<long> v{[] { const char *e = getenv("HSA_CROSS_LEVEL_ROWS_LIMIT"); return e ? atol(e) : 8192L; }()};
+    static std::atomic<long> v{[] { const char *e = getenv("HSA_CROSS_LEVEL_ROWS_LIMIT"); return e ? atol(e) : 0L; }()};
     return v;
+}
+
+// whether the kernel with the head's weights resident in LDS is built for this head layout
+static bool level_pw_capable(int H, int Dh) {
+    const long Dm = (long)H * Dh;
+    return Dh <= 64 && 2 * (Dm / 32) * (Dh / 16) * 1024 <= 128 * 1024;
 }
 
 constexpr int LEVEL_WG_WAVES = 4;
@@ -567,6 +726,46 @@ int launch_level_wg(const TopParams &p, int C, int row, const uint16_t *lsrc, in
     return HSA_OK;
 }
 
+// the variant with the head's weights resident in LDS: where they fit and a workgroup has at
+// least two groups of 16 row tiles to walk
+template <typename T, int CT2>
+int launch_level_pw(const TopParams &p, int C, int row, const uint16_t *lsrc, int64_t lbs, int64_t lrs, hipStream_t st,
+                    bool &taken) {
+    taken = false;
+    const int NK = p.Dm / 32;
+    const size_t lds = (size_t)2 * NK * CT2 * 1024;
+    if (!level_pw_capable(p.H, 16 * CT2)) return HSA_OK;
+    const long tiles = (C + 15) / 16, groups = (tiles + 15) / 16, bh = (long)p.B * p.H;
+    long parts = 256 / bh;
+    if (parts < 1) parts = 1;
+    if (parts > groups) parts = groups;
+    if (groups < 2 * parts) return HSA_OK;
+    if constexpr (CT2 > 4) return HSA_OK;
+    taken = true;
+    auto launch = [&](auto kern) -> int {
+        static std::atomic<bool> allowed[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(HSA_ERR_LAUNCH, "no current device");
+        if (lds > 64 * 1024 && !allowed[dev].load(std::memory_order_acquire)) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            if (e != hipSuccess) return fail(HSA_ERR_LAUNCH, "LDS size %zu refused: %s", lds, hipGetErrorString(e));
+            allowed[dev].store(true, std::memory_order_release);
+        }
+        kern<<<dim3((unsigned)p.B, (unsigned)p.H, (unsigned)parts), 512, lds, st>>>(p, C, row, lsrc, lbs, lrs);
+        return HSA_OK;
+    };
+    if constexpr (CT2 <= 2) {
+        if (NK % 8 == 0) return launch(cross_update_level_pw_kernel<T, CT2, 8>);
+    }
+    if constexpr (CT2 <= 4) {
+        return launch(cross_update_level_pw_kernel<T, CT2, 4>);
+    } else {
+        taken = false;  // 128 channels per head: the accumulators of both halves do not fit two wavefronts per SIMD
+        return HSA_OK;
+    }
+}
+
 // Which variant: two row tiles per wavefront where that still starts a workgroup per CU (else
 // one); two workgroups per CU (chunks of four k-steps: 64 KB of LDS) where there are at least two
 // per CU to start.  Measured at B8 H8 Dh64 (us per level of 4096 / 2048 / 1024 / 512 / 256 / 128
@@ -576,6 +775,11 @@ template <typename T, int CT2>
 int launch_level_wg_any(const TopParams &p, int C, int row, const uint16_t *lsrc, int64_t lbs, int64_t lrs, hipStream_t st) {
     const int NK = p.Dm / 32;
     const long tiles = (C + 15) / 16, bh = (long)p.B * p.H;
+    {
+        bool taken = false;
+        const int rc = launch_level_pw<T, CT2>(p, C, row, lsrc, lbs, lrs, st, taken);
+        if (taken || rc != HSA_OK) return rc;
+    }
     auto wgs = [&](int rt) { return bh * ((tiles + LEVEL_WG_WAVES * rt - 1) / (LEVEL_WG_WAVES * rt)); };
     if constexpr (CT2 <= 4) {
         if (wgs(2) >= 512) return launch_level_wg<T, CT2, 2, 4, 2>(p, C, row, lsrc, lbs, lrs, st);
@@ -667,7 +871,7 @@ int hsa_cross_update_top_tune(int single_launch) {
 }
 
 int hsa_cross_update_level_tune(int wg_min_tiles, long rows_limit) {
-    if (wg_min_tiles < -1 || rows_limit < -1) return hsa::fail(HSA_ERR_INVALID, "negative knob");
+    if (wg_min_tiles < -1 || rows_limit < -1) return hsa::fail(HSA_ERR_INVALID, "knob below -1");
     if (wg_min_tiles >= 0) hsa::level_wg_min_tiles().store(wg_min_tiles);
     if (rows_limit >= 0) hsa::level_rows_limit().store(rows_limit);
     return HSA_OK;
@@ -686,8 +890,13 @@ int hsa_cross_update_level_rows(int B, int H, int Dh, int dtype) {
     // parent build per level while the batch's rows of a level are few (measured on the LM forward
     // at 4096 tokens: up to 4096 rows at batch 1, 1024 at 4, 512 at 8, no gain from 32 on)
     int rows = held;
-    const long limit = hsa::level_rows_limit().load();
-    while ((long)B * rows * 2 <= limit) rows *= 2;
+    // Measured on the LM forward at 4096 tokens, batch 8, 8 heads of 64 channels (us per level of
+    // 4096 / 2048 / 1024 children): a GEMM plus the parent build 71 / 36 / 26, the fused level with
+    // the weights resident in LDS 51 / 29 / -, with the weights staged in chunks 68 / 34 / 18.5:
+    // where the resident variant is built every level is handed over, elsewhere B * C <= 8192.
+    long limit = hsa::level_rows_limit().load();
+    if (limit <= 0) limit = hsa::level_pw_capable(H, Dh) ? (1L << 40) : 8192L;
+    while ((long)B * rows * 2 <= limit && rows * 2 <= (1 << 20)) rows *= 2;
     return rows;
 }
 

@@ -370,20 +370,31 @@ def test_cross_update_top_many_rows_per_level_launches(B, C, H, Dh, top_knob):
     lib = _lib.lib()
     assert lib.hsa_cross_update_level_rows(B, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
     top_knob(0)
-    assert lib.hsa_cross_update_level_rows(1, H, Dh, _lib.HSA_BF16) == 8192
-    assert lib.hsa_cross_update_level_rows(8, H, Dh, _lib.HSA_BF16) == 1024
-    assert lib.hsa_cross_update_level_rows(4096, H, Dh, _lib.HSA_BF16) == fn.fused_top_rows(H, Dh, torch.bfloat16)
+    # heads whose weights fit the LDS hand every level over; 128-channel heads while B * C <= 8192
+    assert lib.hsa_cross_update_level_rows(1, 8, 64, _lib.HSA_BF16) == 1 << 20
+    assert lib.hsa_cross_update_level_rows(8, 8, 64, _lib.HSA_BF16) == 1 << 20
+    assert lib.hsa_cross_update_level_rows(8, 16, 64, _lib.HSA_BF16) == 1024     # 256 KiB of weights per head
+    assert lib.hsa_cross_update_level_rows(1, 4, 128, _lib.HSA_BF16) == 8192
+    assert lib.hsa_cross_update_level_rows(8, 4, 128, _lib.HSA_BF16) == 1024
+    assert lib.hsa_cross_update_level_tune(-1, 4096) == 0
+    assert lib.hsa_cross_update_level_rows(8, 8, 64, _lib.HSA_BF16) == 512
+    assert lib.hsa_cross_update_level_tune(-1, 0) == 0
+    assert lib.hsa_cross_update_level_rows(4096, 4, 128, _lib.HSA_BF16) == fn.fused_top_rows(4, 128, torch.bfloat16)
     assert lib.hsa_cross_update_level_rows(1, 3, 24, _lib.HSA_BF16) == 0
 
 
 @pytest.mark.parametrize("B,C,H,Dh", [(8, 1024, 8, 64), (8, 512, 8, 64), (2, 1024, 8, 64), (16, 256, 4, 32), (4, 512, 2, 128),
-                                      (8, 256, 6, 64), (3, 128, 4, 64)])
+                                      (8, 256, 6, 64), (3, 128, 4, 64),
+                                      # several groups of row tiles per workgroup, the weights resident in LDS
+                                      (8, 2048, 8, 64), (16, 1024, 8, 64), (6, 4096, 8, 64), (2, 4096, 6, 64), (4, 2048, 8, 32)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_cross_update_levels_weights_staged_per_workgroup(B, C, H, Dh, dtype):
-    """Large levels run on the kernel that stages a head's weights in LDS once per workgroup (two
-    row tiles per wavefront or one, one or two workgroups per CU, chunks of four or eight k-steps,
-    a model width that is no multiple of 256): bit-identical to the launch per wavefront and row
-    tile, which rounds at the same places, and close to the level-by-level kernels."""
+    """Large levels run on the kernels that keep a head's weights in LDS (staged in chunks per
+    workgroup: two row tiles per wavefront or one, one or two workgroups per CU, chunks of four or
+    eight k-steps, a model width that is no multiple of 256; or resident while a workgroup walks
+    several groups of row tiles, an uneven share of groups included): bit-identical to the launch
+    per wavefront and row tile, which rounds at the same places, and close to the level-by-level
+    kernels."""
     dim = H * Dh
     g = torch.Generator().manual_seed(C + H + B)
     src = torch.randn(B, C, dim, generator=g).clamp(-1, 1).to(dtype).to(DEV)
