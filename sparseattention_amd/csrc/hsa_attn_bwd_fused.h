@@ -12,8 +12,9 @@
 // state instead of being exchanged: the neighbour's Q and dO rows, the forward's log-sum-exp of
 // those queries (P = exp2(logit - lse)) and delta = <dO, O> from the forward's output rows.
 // So every row of Q, dO, K, V is fetched once per strip plus one halo block per strip (or two),
-// nothing leaves as a partial result except the rows of levels >= 6 (one fp32 row per 64 queries
-// and level, summed by a small second launch), and there are no atomics.
+// nothing leaves as a partial result except the rows of the levels whose nodes collect from more
+// than one strip (from level 7 with strips of four blocks, from level 8 with strips of eight: one
+// fp32 row per strip and level, summed by a small second launch), and there are no atomics.
 //
 // What it costs: a wavefront carries the waiting key blocks' accumulators on top of everything the
 // query pass holds: 300-360 registers at 64 channels per head, i.e. one wavefront per SIMD (two at
@@ -641,23 +642,40 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             }
         }
 
-        // levels >= 6: partial rows, laid out per run of four blocks.  Level 6: the run that ends
-        // here; the levels above: the strip, stored with its last block in the strip's first run
+        // levels >= 6.  A level-6 node collects from the run of four blocks under its sibling, a
+        // level-7 node from the eight blocks of a strip: those rows are final when the run (the
+        // strip of eight) ends here and go straight to dK / dV (zeros where the causal mask leaves
+        // the node to nobody: the probabilities were zero).  The levels above have several strips
+        // under the sibling: partial rows, laid out per run of four blocks and stored with the
+        // strip's last block in the strip's first run, summed by the second launch.
         if ((it & (FAR - 1)) == FAR - 1) {
+            constexpr int LVF = SB == 8 ? 7 : 6;  // the highest level a strip finishes alone
             const int lvl = 6 + r16;
             const int LF = L - 6;
             if (lvl < L && (it == SB - 1 || r16 == 0)) {
-                const int NR = NB / FAR;
-                float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
-                const int run = r16 == 0 ? blk / FAR : blk0 / FAR;
-                const size_t po = ((((size_t)b * NR + run) * H + h) * LF + (lvl - 6)) * D;
-                float *pkp = far + po + half * HD;
-                float *pvp = far + (size_t)p.B * NR * H * LF * D + po + half * HD;
+                if (lvl <= LVF) {
+                    const int node = (lvl == 6 ? blk / FAR : blk0 / SB) ^ 1;
+                    const size_t ro = ko + (size_t)(level_offset(N, lvl) + node) * rs;
 #pragma unroll
-                for (int j = 0; j < NJ; ++j) {
-                    const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
-                    *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
-                    *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
+                    for (int j = 0; j < NJ; ++j) {
+                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                        *reinterpret_cast<u32x2_t *>(p.dk + ro + ch) =
+                            u32x2_t{M_::pack(fk[j][0], fk[j][1]), M_::pack(fk[j][2], fk[j][3])};
+                        *reinterpret_cast<u32x2_t *>(p.dv + ro + ch) =
+                            u32x2_t{M_::pack(fv[j][0], fv[j][1]), M_::pack(fv[j][2], fv[j][3])};
+                    }
+                } else {
+                    const int NR = NB / FAR;
+                    float *far = p.partial + 2 * (size_t)p.B * NB * H * 2 * D;
+                    const size_t po = ((((size_t)b * NR + blk0 / FAR) * H + h) * LF + (lvl - 6)) * D;
+                    float *pkp = far + po + half * HD;
+                    float *pvp = far + (size_t)p.B * NR * H * LF * D + po + half * HD;
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+                        const int ch = 32 * (j >> 1) + 8 * g + 4 * (j & 1);
+                        *reinterpret_cast<f32x4 *>(pkp + ch) = fk[j];
+                        *reinterpret_cast<f32x4 *>(pvp + ch) = fv[j];
+                    }
                 }
             }
         }
@@ -705,8 +723,9 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     }
 }
 
-// the rows of levels >= 6 (and the root row, the rows nobody attends, the rows past 2N-1) from the
-// strips' partial rows
+// the rows of the levels no strip finishes alone (from level 7 with strips of four blocks, from
+// level 8 with strips of eight; and the root row, the rows nobody attends, the rows past 2N-1) from
+// the strips' partial rows
 template <typename T>
 __global__ void __launch_bounds__(BWD_WPB * 64) attn_bwd_reduce_kernel(BwdTileParams p, int D) {
     using S = typename T::storage;
@@ -743,6 +762,13 @@ static int bwd_fused_launch_one(const BwdFusedParams &q, hipStream_t st) {
         if (nbw == 2 && !causal) return fail(HSA_ERR_UNSUPPORTED, "one-pass backward: window radius above 16 needs the causal mask"); \
         q.t.n_units = fp.t.n_units / sb;                                                                    \
         q.t.red_lg_sb = sb == 8 ? 3 : 2;                                                                    \
+        {   /* the second launch starts above the levels the strips finish themselves */                    \
+            int first = level_offset(fp.t.N, sb == 8 ? 8 : 7);                                              \
+            if (first > 2 * fp.t.N - 2) first = 2 * fp.t.N - 2;                                             \
+            const size_t threads = (size_t)fp.t.B * (fp.t.M - first) * fp.t.H * (D / 4) * BWD_FUSED_RED_SPLIT; \
+            q.t.red_first_row = first;                                                                      \
+            q.t.red_wgs = (int)((threads + BWD_WPB * 64 - 1) / (BWD_WPB * 64));                             \
+        }                                                                                                   \
         int rc;                                                                                             \
         if (nbw == 2) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 2>(q, st) : bwd_fused_launch_one<T, D, true, 4, 2>(q, st); \
         else if (causal) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 1>(q, st) : bwd_fused_launch_one<T, D, true, 4, 1>(q, st); \

@@ -790,8 +790,9 @@ static int attn_bwd_fused_typed(const void *q, const void *k, const void *v, con
     p.n_units = (int)units;
     p.scale = 1.0f / sqrtf((float)D);
     p.scale_log2e = 1.4426950408889634f * p.scale;
-    // the strips finish levels 1..5; the rows above them, the root row and the rows past 2N-1 are
-    // summed from the strips' partial rows by a second, small launch
+    // the strips finish levels 1..6 (..7 with strips of eight blocks); the rows above them, the root
+    // row and the rows past 2N-1 are summed from the strips' partial rows by a second, small
+    // launch, whose first row the launcher sets once it knows the strip length
     int first = level_offset(N, 6);
     if (first > 2 * N - 2) first = 2 * N - 2;
     const size_t red_threads = (size_t)B * (M - first) * H * (D / 4) * BWD_FUSED_RED_SPLIT;
