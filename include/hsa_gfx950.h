@@ -334,7 +334,9 @@ int hsa_attn_bwd_saved(const void *q, const void *k, const void *v, const void *
  * Query blocks one wavefront of hsa_attn_bwd_saved walks (no counterpart in the reference; for
  * experiments and tests, results do not depend on it beyond rounding): 0 = automatic (eight where
  * that many wavefronts still fill the chip, 64 channels per head and the sequence has a multiple
- * of eight blocks; else four), 4, or 8 (used where the sequence allows it).  Process-wide.
+ * of eight blocks; 16 or 32 where that still leaves four rounds of wavefronts; else four), or 4,
+ * 8, 16, 32 (the largest of these up to the argument that divides the sequence's block count).
+ * Process-wide.
  */
 int hsa_attn_bwd_saved_tune(int strip_blocks);
 

@@ -13,7 +13,7 @@
 // those queries (P = exp2(logit - lse)) and delta = <dO, O> from the forward's output rows.
 // So every row of Q, dO, K, V is fetched once per strip plus one halo block per strip (or two),
 // nothing leaves as a partial result except the rows of the levels whose nodes collect from more
-// than one strip (from level 7 with strips of four blocks, from level 8 with strips of eight: one
+// than one strip (from level 7 with strips of four blocks, level 8 with eight, ... level 10 with 32: one
 // fp32 row per strip and level, summed by a small second launch), and there are no atomics.
 //
 // What it costs: a wavefront carries the waiting key blocks' accumulators on top of everything the
@@ -27,9 +27,10 @@
 // instruction time is what is left to hide behind the memory system.
 // Requesting two blocks ahead (into the area whose operands have just left for the registers) is
 // slower: 52.4 us.
-// Strips of eight blocks where that still fills every wavefront slot: one neighbour's block per
-// 128 queries instead of per 64 (the far tree block and its partial rows change in the middle of
-// the strip, the leaf key blocks' accumulators just carry on).
+// Strips of 8, 16 or 32 blocks where that still fills every wavefront slot: one neighbour's block
+// per 128 .. 512 queries instead of per 64, and the tree levels whose nodes collect from up to that
+// many queries are final inside the strip (the far tree block changes every four blocks, the leaf
+// key blocks' accumulators just carry on).
 #pragma once
 
 #include "hsa_attn_bwd_tile.h"
@@ -61,7 +62,7 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     constexpr int WPB = SPLIT == 2 ? 2 : BWD_WPB;       // wavefronts per workgroup
     using BT = BwdTile<T, HD>;
     using M_ = Mma<T>;
-    static_assert(SB == 4 || SB == 8, "a strip is one or two runs of four blocks (the 64 leaves under a level-6 node)");
+    static_assert(SB == 4 || SB == 8 || SB == 16 || SB == 32, "a strip is 1, 2, 4 or 8 runs of four blocks (the 64 leaves under a level-6 node)");
     static_assert(NBW == 1 || (NBW == 2 && CAUSAL), "window radius up to 16, or up to 32 with the causal mask");
     constexpr int FAR = BWD_STRIP;  // blocks that share the far tree block
     constexpr int KS = BT::KS, NJ = BT::NJ, RPI = BT::RPI, NLD = BT::NLD, CPR = BT::CPR;
@@ -400,9 +401,9 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             bt.get(0, Kc[NKL + 1]);
             bt.get(1, Vc[NKL + 1]);
             far_biases(q0);
-            // the strip's second run goes on summing the levels above 6, whose nodes it shares
-            // with the first; level 6 (the lanes of slot 0) starts over
-            if (it == 0 || r16 == 0) {
+            // a later run of the strip goes on summing the levels whose nodes it shares with the
+            // runs before: slot r16 (level 6 + r16) starts over every 4 << r16 blocks
+            if ((it & ((4 << r16) - 1)) == 0) {
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) { fk[j] = f32x4{0.f, 0.f, 0.f, 0.f}; fv[j] = f32x4{0.f, 0.f, 0.f, 0.f}; }
             }
@@ -642,19 +643,19 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
             }
         }
 
-        // levels >= 6.  A level-6 node collects from the run of four blocks under its sibling, a
-        // level-7 node from the eight blocks of a strip: those rows are final when the run (the
-        // strip of eight) ends here and go straight to dK / dV (zeros where the causal mask leaves
-        // the node to nobody: the probabilities were zero).  The levels above have several strips
-        // under the sibling: partial rows, laid out per run of four blocks and stored with the
-        // strip's last block in the strip's first run, summed by the second launch.
+        // levels >= 6.  The node of level 6 + r collects from the 4 << r blocks under its sibling:
+        // where the strip holds all of them (level 6: a run of four blocks, level 7: eight, ...) the
+        // row is final when the last of them ends here and goes straight to dK / dV (zeros where
+        // the causal mask leaves the node to nobody: the probabilities were zero).  The levels above
+        // have several strips under the sibling: partial rows, laid out per run of four blocks and
+        // stored with the strip's last block in the strip's first run, summed by the second launch.
         if ((it & (FAR - 1)) == FAR - 1) {
-            constexpr int LVF = SB == 8 ? 7 : 6;  // the highest level a strip finishes alone
             const int lvl = 6 + r16;
             const int LF = L - 6;
-            if (lvl < L && (it == SB - 1 || r16 == 0)) {
-                if (lvl <= LVF) {
-                    const int node = (lvl == 6 ? blk / FAR : blk0 / SB) ^ 1;
+            const bool final_row = ((it + 1) & ((4 << r16) - 1)) == 0;  // never for 4 << r16 > SB
+            if (lvl < L && (final_row || it == SB - 1)) {
+                if (final_row) {
+                    const int node = (blk >> (lvl - 4)) ^ 1;
                     const size_t ro = ko + (size_t)(level_offset(N, lvl) + node) * rs;
 #pragma unroll
                     for (int j = 0; j < NJ; ++j) {
@@ -723,9 +724,9 @@ attn_bwd_tile_fused_kernel(BwdFusedParams fp) {
     }
 }
 
-// the rows of the levels no strip finishes alone (from level 7 with strips of four blocks, from
-// level 8 with strips of eight; and the root row, the rows nobody attends, the rows past 2N-1) from
-// the strips' partial rows
+// the rows of the levels no strip finishes alone (from level 7 with strips of four blocks up to
+// from level 10 with strips of 32; and the root row, the rows nobody attends, the rows past 2N-1)
+// from the strips' partial rows
 template <typename T>
 __global__ void __launch_bounds__(BWD_WPB * 64) attn_bwd_reduce_kernel(BwdTileParams p, int D) {
     using S = typename T::storage;
@@ -749,30 +750,45 @@ static int bwd_fused_launch_one(const BwdFusedParams &q, hipStream_t st) {
     return check_launch("attn_bwd_tile_fused_kernel");
 }
 
+template <typename T, int D, bool CAUSAL, int NBW>
+static int bwd_fused_launch_sb(const BwdFusedParams &q, int sb, hipStream_t st) {
+    switch (sb) {
+        case 32: return bwd_fused_launch_one<T, D, CAUSAL, 32, NBW>(q, st);
+        case 16: return bwd_fused_launch_one<T, D, CAUSAL, 16, NBW>(q, st);
+        case 8: return bwd_fused_launch_one<T, D, CAUSAL, 8, NBW>(q, st);
+        default: return bwd_fused_launch_one<T, D, CAUSAL, 4, NBW>(q, st);
+    }
+}
+
 #define HSA_BWD_FUSED_INSTANTIATE(T, D)                                                                     \
     template <>                                                                                             \
     int attn_bwd_fused_launch_td<T, D>(const BwdFusedParams &fp, bool causal, hipStream_t st) {             \
         BwdFusedParams q = fp;                                                                              \
         const int NB = fp.t.N / TILE_Q;                                                                     \
-        /* strips of eight where their wavefronts still fill the chip (one per SIMD on 256 CUs) */          \
+        /* the longest strips (8, 16, 32 blocks) whose wavefronts still fill the chip once (one per SIMD */ \
+        /* on 256 CUs): fewer halo blocks, more tree levels final inside the strip.  Measured (us, strips */ \
+        /* of 8 / 16 / 32): B8 H8 N4096 D64 93 / 88 / 119, B8 H8 N8192 D64 180 / 173 / 166, B1 H16 N65536 */ \
+        /* D64 348 / 327 / 317, B1 H16 N65536 D128 R32 734 / 679 / 657, B1 H16 N16384 D64 92.6 / 94.2 / 120 */ \
         const long waves8 = (long)(fp.t.n_units / 8) * (D > 64 ? 2 : 1);                                    \
         const int knob = bwd_fused_strip_knob();                                                            \
-        const int sb = (NB % 8 == 0 && knob != 4 && (knob == 8 || (D >= 64 && waves8 >= 1024))) ? 8 : 4;    \
+        int sb = (NB % 8 == 0 && knob != 4 && (knob >= 8 || (D >= 64 && waves8 >= 1024))) ? 8 : 4;          \
+        if (sb == 8 && NB % 16 == 0 && (knob >= 16 || (knob == 0 && waves8 >= 2 * 1024))) sb = 16;          \
+        if (sb == 16 && NB % 32 == 0 && (knob >= 32 || (knob == 0 && waves8 >= 4 * 1024))) sb = 32;         \
         const int nbw = fp.t.R > TILE_Q ? 2 : 1;                                                            \
         if (nbw == 2 && !causal) return fail(HSA_ERR_UNSUPPORTED, "one-pass backward: window radius above 16 needs the causal mask"); \
         q.t.n_units = fp.t.n_units / sb;                                                                    \
-        q.t.red_lg_sb = sb == 8 ? 3 : 2;                                                                    \
+        q.t.red_lg_sb = sb == 32 ? 5 : sb == 16 ? 4 : sb == 8 ? 3 : 2;                                      \
         {   /* the second launch starts above the levels the strips finish themselves */                    \
-            int first = level_offset(fp.t.N, sb == 8 ? 8 : 7);                                              \
+            int first = level_offset(fp.t.N, q.t.red_lg_sb + 5);                                            \
             if (first > 2 * fp.t.N - 2) first = 2 * fp.t.N - 2;                                             \
             const size_t threads = (size_t)fp.t.B * (fp.t.M - first) * fp.t.H * (D / 4) * BWD_FUSED_RED_SPLIT; \
             q.t.red_first_row = first;                                                                      \
             q.t.red_wgs = (int)((threads + BWD_WPB * 64 - 1) / (BWD_WPB * 64));                             \
         }                                                                                                   \
         int rc;                                                                                             \
-        if (nbw == 2) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 2>(q, st) : bwd_fused_launch_one<T, D, true, 4, 2>(q, st); \
-        else if (causal) rc = sb == 8 ? bwd_fused_launch_one<T, D, true, 8, 1>(q, st) : bwd_fused_launch_one<T, D, true, 4, 1>(q, st); \
-        else rc = sb == 8 ? bwd_fused_launch_one<T, D, false, 8, 1>(q, st) : bwd_fused_launch_one<T, D, false, 4, 1>(q, st); \
+        if (nbw == 2) rc = bwd_fused_launch_sb<T, D, true, 2>(q, sb, st);                                   \
+        else if (causal) rc = bwd_fused_launch_sb<T, D, true, 1>(q, sb, st);                                \
+        else rc = bwd_fused_launch_sb<T, D, false, 1>(q, sb, st);                                           \
         if (rc != HSA_OK || q.t.red_wgs == 0) return rc;                                                    \
         attn_bwd_reduce_kernel<T><<<q.t.red_wgs, BWD_WPB * 64, 0, st>>>(q.t, D);                            \
         return check_launch("attn_bwd_reduce_kernel");                                                      \

@@ -751,12 +751,12 @@ __device__ __forceinline__ void bwd_reduce_rows(const float *__restrict__ partia
                 pk = partial + (((size_t)b * NB + blk0) * H + h) * 2 * D + (size_t)(lvl - 4) * D + d;
                 pv = pk + (size_t)B * NB * H * 2 * D;
             } else {
-                // lg_sb == 3 (the one-pass variant's strips of eight blocks): the area is laid out per
+                // lg_sb >= 3 (the one-pass variant's strips of eight or more blocks): the area is laid out per
                 // run of four blocks; level 6 has a row per run, the levels above one per strip, in
                 // the strip's first run
                 const int LF = L - 6;
-                const int lgl = lg_sb == 3 ? 2 : lg_sb;             // layout granularity
-                const int lg = (lg_sb == 3 && lvl == 6) ? 2 : lg_sb;  // blocks summed into one row
+                const int lgl = lg_sb >= 3 ? 2 : lg_sb;             // layout granularity
+                const int lg = (lg_sb >= 3 && lvl == 6) ? 2 : lg_sb;  // blocks summed into one row
                 const int NR = NB >> lgl;
                 n = (1 << (lvl - 4)) >> lg;
                 stride = ((size_t)H * LF * D) << (lg - lgl);

@@ -926,8 +926,8 @@ int hsa_attn_bwd_tables(const void *q, const void *k, const void *v, const void 
 }
 
 int hsa_attn_bwd_saved_tune(int strip_blocks) {
-    if (strip_blocks != 0 && strip_blocks != 4 && strip_blocks != 8)
-        return hsa::fail(HSA_ERR_INVALID, "strip length %d (0, 4 or 8)", strip_blocks);
+    if (strip_blocks != 0 && strip_blocks != 4 && strip_blocks != 8 && strip_blocks != 16 && strip_blocks != 32)
+        return hsa::fail(HSA_ERR_INVALID, "strip length %d (0, 4, 8, 16 or 32)", strip_blocks);
     hsa::bwd_fused_strip_knob() = strip_blocks;
     return HSA_OK;
 }

@@ -1174,7 +1174,8 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
     two = fn.attention_backward(gd, qd, kd, vd, R, causal)
     # strips of four and of eight query blocks per wavefront (eight: one neighbour's block per 128
     # queries, the far tree block changes in the middle of the strip)
-    for strip in (4, 8):
+    # (16 and 32: long sequences; more tree levels are final inside the strip)
+    for strip in (4, 8, 16, 32):
         assert _lib.lib().hsa_attn_bwd_saved_tune(strip) == 0
         try:
             forced = fn.attention_backward_saved(gd, qd, kd, vd, out, lse, R, causal)
@@ -1270,6 +1271,25 @@ def test_attention_backward_long_sequence_upper_levels(causal):
     assert (tile[0].float() - gath[0].float()).abs().max() <= 3e-2 * max(1.0, float(gath[0].float().abs().max()))
     # the root row is attended by nobody
     assert not tile[1][:, 2 * N - 2].any() and not tile[2][:, 2 * N - 2].any()
+    # the one-pass formulation with its automatic strip length and with strips of 16 and 32 query
+    # blocks (levels up to 8 / 9 finished inside a strip, the rest from partial rows)
+    out, lse = fn.attention_forward_lse(q, k, v, R, causal)
+    for knob in (0, 16, 32):
+        assert _lib.lib().hsa_attn_bwd_saved_tune(knob) == 0
+        try:
+            one = fn.attention_backward_saved(go, q, k, v, out, lse, R, causal)
+        finally:
+            _lib.lib().hsa_attn_bwd_saved_tune(0)
+        off = N
+        for lvl in range(1, N.bit_length()):
+            rows = N >> lvl
+            for a, b, name in ((one[1], gath[1], "dK"), (one[2], gath[2], "dV")):
+                x, y = a[:, off:off + rows].float(), b[:, off:off + rows].float()
+                scale = max(1.0, float(y.abs().max()))
+                assert (x - y).abs().max() <= 3e-2 * scale, "one pass, knob %d: %s level %d (scale %.1f)" % (knob, name, lvl, scale)
+            off += rows
+        assert (one[0].float() - gath[0].float()).abs().max() <= 3e-2 * max(1.0, float(gath[0].float().abs().max()))
+        assert not one[1][:, 2 * N - 2].any() and not one[2][:, 2 * N - 2].any()
 
 
 def test_attention_backward_unknown_tables_need_their_gather_table():
