@@ -449,6 +449,48 @@ def copy_reference(torch, stream, K, nbytes):
     return e0.elapsed_time(e1) / K, 2 * half
 
 
+def backward_times(torch, _lib, lib, prob, stream, st, K, causal):
+    """Average time of the span attention backward on the problem's rotated inputs, both
+    launches of each formulation between one pair of events: (two passes, one pass on the saved
+    forward state or None where that is not built)."""
+    B, H, N, D, R = prob.B, prob.H, prob.N, prob.D, prob.R
+    M, L = 2 * N - 1, N.bit_length() - 1
+    dev = prob.sets[0]["q"].device
+    nsets = len(prob.sets)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    s0 = prob.sets[0]
+    gq = torch.randn(B, N, H, D, device=dev).to(torch.bfloat16)
+    dq_, dk_, dv_ = torch.empty_like(gq), torch.empty_like(s0["kfull"]), torch.empty_like(s0["kfull"])
+    wsb = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.HSA_BF16, _lib.ATTN_AUTO))
+    wsp = torch.empty(max(wsb, 4) // 4 + 1, device=dev, dtype=torch.float32)
+    bargs = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(gq), P(dq_), P(dk_), P(dv_), P(wsp), wsp.numel() * 4,
+              B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st) for s in prob.sets]
+    for i in range(3):
+        assert lib.hsa_attn_bwd(*bargs[i % nsets]) == 0, lib.hsa_last_error()
+    two_ms = median(repeated(
+        lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd(*bargs[i % nsets])), K, min_reps=7,
+        min_total_ms=6.0))
+    # the one-pass backward on saved forward state, where it is built
+    one_ms = None
+    if int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16)) > 0:
+        saved = []
+        for s in prob.sets:
+            o_ = torch.empty_like(s["q"])
+            lse_ = torch.empty(B, N, H, device=dev, dtype=torch.float32)
+            assert lib.hsa_attn_fwd_lse(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), B, N, M, H, D, L, R,
+                                        int(causal), _lib.HSA_BF16, st) == 0, lib.hsa_last_error()
+            saved.append((o_, lse_))
+        b1args = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), P(gq), P(dq_), P(dk_), P(dv_), P(wsp),
+                   wsp.numel() * 4, B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, st)
+                  for s, (o_, lse_) in zip(prob.sets, saved)]
+        for i in range(3):
+            assert lib.hsa_attn_bwd_saved(*b1args[i % nsets]) == 0, lib.hsa_last_error()
+        one_ms = median(repeated(
+            lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd_saved(*b1args[i % nsets])), K,
+            min_reps=7, min_total_ms=6.0))
+    return two_ms, one_ms
+
+
 def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
     """Kernel times, GB/s and fraction of the HBM peak of one configuration, its one-stream step
     time, and its CPU baseline on a bounded sample."""
@@ -478,6 +520,13 @@ def brief_config(torch, _lib, lib, hip, name, causal, K, cpu_seconds):
            "single_stream_head_queries_per_s": prob.head_queries / (step_ms * 1e-3),
            "device_copy_of_attn_bytes_ms": copy_reference(torch, stream, K, prob.attn_bytes)[0],
            "device_copy_of_tree_bytes_ms": copy_reference(torch, stream, K, prob.tree_bytes)[0]}
+    two_ms, one_ms = backward_times(torch, _lib, lib, prob, stream, st, K, causal)
+    bwd_bytes = 2 * B * H * D * (3 * N + 4 * (2 * N - 1))  # Q, dO, dQ and K, V, dK, dV once each
+    rec["attn_backward_avg_ms"] = two_ms
+    rec["attn_backward_one_pass_avg_ms"] = one_ms
+    rec["attn_backward_algorithmic_bytes"] = bwd_bytes
+    best = min(two_ms, one_ms) if one_ms is not None else two_ms
+    rec["attn_backward_frac_of_hbm_peak"] = bwd_bytes / (best * 1e-3) / 1e9 / HBM_PEAK_GBS
     del prob
     torch.cuda.empty_cache()
     if cpu_seconds > 0:
@@ -557,39 +606,7 @@ def main():
     attn_event_avg_ms = sum(attn_kernel_ms) / K
 
     # --- backward of the span attention (next-row kernel), same rotation of inputs ----------------
-    P = lambda t: ctypes.c_void_p(t.data_ptr())
-    s0 = prob.sets[0]
-    gq = torch.randn(B, N, H, D, device=dev).to(torch.bfloat16)
-    dq_, dk_, dv_ = torch.empty_like(gq), torch.empty_like(s0["kfull"]), torch.empty_like(s0["kfull"])
-    wsb = int(lib.hsa_attn_bwd_workspace_bytes(B, N, M, H, D, L, R, _lib.HSA_BF16, _lib.ATTN_AUTO))
-    wsp = torch.empty(max(wsb, 4) // 4 + 1, device=dev, dtype=torch.float32)
-    bargs = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(gq), P(dq_), P(dk_), P(dv_), P(wsp), wsp.numel() * 4,
-              B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, _lib.ATTN_AUTO, st) for s in prob.sets]
-    for i in range(3):
-        assert lib.hsa_attn_bwd(*bargs[i % nsets]) == 0, lib.hsa_last_error()
-    attn_bwd_ms = median(repeated(
-        lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd(*bargs[i % nsets])), K, min_reps=7,
-        min_total_ms=6.0))
-    # the one-pass backward on saved forward state (opt-in: less traffic, more time), where it applies
-    attn_bwd1_ms = None
-    if int(lib.hsa_attn_bwd_saved_workspace_bytes(B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16)) > 0:
-        saved = []
-        for s in prob.sets:
-            o_ = torch.empty_like(s["q"])
-            lse_ = torch.empty(B, N, H, device=dev, dtype=torch.float32)
-            assert lib.hsa_attn_fwd_lse(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), B, N, M, H, D, L, R,
-                                        int(causal), _lib.HSA_BF16, st) == 0, lib.hsa_last_error()
-            saved.append((o_, lse_))
-        b1args = [(P(s["q"]), P(s["kfull"]), P(s["vfull"]), P(o_), P(lse_), P(gq), P(dq_), P(dk_), P(dv_), P(wsp),
-                   wsp.numel() * 4, B, N, M, H, D, L, R, int(causal), _lib.HSA_BF16, st)
-                  for s, (o_, lse_) in zip(prob.sets, saved)]
-        for i in range(3):
-            assert lib.hsa_attn_bwd_saved(*b1args[i % nsets]) == 0, lib.hsa_last_error()
-        attn_bwd1_ms = median(repeated(
-            lambda: between_events(torch, stream, K, lambda i: lib.hsa_attn_bwd_saved(*b1args[i % nsets])), K,
-            min_reps=7, min_total_ms=6.0))
-        del saved, b1args
-    del gq, dq_, dk_, dv_, wsp
+    attn_bwd_ms, attn_bwd1_ms = backward_times(torch, _lib, lib, prob, stream, st, K, causal)
 
     # --- reference point: a plain device-to-device copy that moves as many bytes as one launch of
     #     the attention kernel (half read, half written), buffers rotated through 1 GiB like the
@@ -650,6 +667,8 @@ def main():
                    "attn_backward_avg_ms": attn_bwd_ms,
                    "attn_backward_one_pass_avg_ms": attn_bwd1_ms,
                    "attn_backward_algorithmic_bytes": E * B * H * D * (2 * N + 2 * M + N + 2 * M),
+                   "attn_backward_frac_of_hbm_peak": E * B * H * D * (2 * N + 2 * M + N + 2 * M) / (
+                       min(attn_bwd_ms, attn_bwd1_ms or attn_bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
                    "device_copy_of_the_same_bytes": {
                        "bytes": copy_bytes, "avg_ms": copy_ms, "GBps": copy_bytes / (copy_ms * 1e-3) / 1e9,
                        "frac_of_hbm_peak": copy_bytes / (copy_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
