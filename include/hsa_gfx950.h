@@ -92,7 +92,8 @@ int hsa_attn_fwd_timed(const void *q, const void *k, const void *v, const int32_
 /*
  * Launch parameters of the 16-bit MFMA tile kernel, for experiments (no counterpart in the
  * reference, whose Triton launch fixes one program per query, ops/functional.py:143-161).
- *   strip_blocks     16-query blocks one wavefront walks: 1, 2 or 4; 0 = chosen by problem size
+ *   strip_blocks     16-query blocks one wavefront walks: 1, 2, 4, or 8 (two runs of four; four
+ *                    where the window radius does not allow runs); 0 = chosen by problem size
  *   waves_per_group  wavefronts per workgroup, 1..8; 0 = chosen by head count (default)
  *   xcd_remap        0 = workgroup ids map to strips in order, 1 = neighbouring strips share an XCD
  *   alternate        0 = every strip walks upwards, 1 = neighbouring strips walk towards each other

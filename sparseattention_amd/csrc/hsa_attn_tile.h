@@ -71,6 +71,7 @@ struct TileParams {
     int B, N, M, H, L, R;
     int NS;       // strips per sequence
     int n_units;  // B * NS * H
+    int runs;     // runs of SB blocks one wavefront walks (a strip is SB * runs blocks): the kernel's RUNS
     int xcd_swizzle;
     int alternate;    // neighbouring strips walk in opposite directions
     float scale_log2e;
@@ -94,10 +95,17 @@ template <int D, int NKL = 1> constexpr int tile_max_wpb() { return (D > 64 || N
 // dead slots zero).  A block's 16 rows of weights are assembled in the wavefront's LDS region
 // (the operand slots are free once the MFMA operands have been read) and written out as
 // whole rows.  Needs 2R+1+L <= D*2+16 floats per row to fit.
-template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false, bool LSE = false>
+// RUNS > 1: a wavefront walks RUNS consecutive runs of SB = 4 blocks (long sequences).  The leaf
+// blocks slide on across the runs, so the neighbouring blocks of the window are fetched once per
+// strip of 4 * RUNS blocks instead of once per four; only the far tree block (the same for the 64
+// queries of a run) is exchanged between runs, requested two blocks ahead.  Straight-line code
+// like a single run; two runs are built.
+template <typename T, int D, int NBW, bool CAUSAL, int SB, bool WT = false, bool LSE = false, int RUNS = 1>
 __global__ void __launch_bounds__((tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>() * 64))
 attn_tile_kernel(TileParams p) {
     using M_ = Mma<T>;
+    constexpr bool MULTI = RUNS > 1;
+    static_assert(!MULTI || (SB == 4 && !WT), "runs are the 64 queries that share a far tree block");
     constexpr int KS = D / 32;                         // 32-channel steps of the QK contraction
     constexpr int NJ = D / 16;                         // 16-channel output tiles
     constexpr int NKL = CAUSAL ? NBW + 1 : 2 * NBW + 1;  // leaf key blocks per query block
@@ -141,7 +149,8 @@ attn_tile_kernel(TileParams p) {
 
     const int N = p.N, L = p.L, R = p.R;
     const int NB = N / TILE_Q;
-    const int blk0 = s * SB;  // NB is a multiple of SB (both powers of two, SB <= NB)
+    constexpr int TOT = SB * RUNS;  // blocks per strip
+    const int blk0 = s * TOT;       // NB is a multiple of the strip length (powers of two, strip <= NB)
     const size_t rs = (size_t)p.H * D;  // elements between consecutive rows
     const uint16_t *Qb = p.q + ((size_t)b * N * p.H + h) * D + 8 * lchk;
     const uint16_t *Kb = p.k + ((size_t)b * p.M * p.H + h) * D + 8 * lchk;
@@ -219,14 +228,15 @@ attn_tile_kernel(TileParams p) {
         }
         biasT[i] = live ? 0.0f : NEG_INF;
     }
-    const int qs = blk0 * TILE_Q;  // first query of the strip
     float biasU[4];
+    auto far_biases = [&](int qs) {  // qs: first query of the run (64 aligned queries)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int lvl = 6 + 4 * g + i;
-        const bool live = lvl < L && (!CAUSAL || ((qs >> lvl) & 1));
-        biasU[i] = live ? 0.0f : NEG_INF;
-    }
+        for (int i = 0; i < 4; ++i) {
+            const int lvl = 6 + 4 * g + i;
+            const bool live = lvl < L && (!CAUSAL || ((qs >> lvl) & 1));
+            biasU[i] = live ? 0.0f : NEG_INF;
+        }
+    };
 
     // ---- loaders: raw[i] = piece lchk of row (i*RPI + lrow) of a 16-row block ---------------
     auto load_block = [&](const uint16_t *base, int row0, u32x4_t (&dst)[NLD], auto nt) {  // consecutive rows
@@ -251,7 +261,7 @@ attn_tile_kernel(TileParams p) {
             if (t_valid[i]) dst[i] = ld16<nt_tree>(base + (size_t)tr * rs);
         }
     };
-    auto load_far = [&](const uint16_t *base, u32x4_t (&dst)[NLD]) {
+    auto load_far = [&](const uint16_t *base, int qs, u32x4_t (&dst)[NLD]) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             dst[i] = u32x4_t{0u, 0u, 0u, 0u};
@@ -300,7 +310,9 @@ attn_tile_kernel(TileParams p) {
     auto run = [&](auto rev_tag) {
     constexpr bool REV = decltype(rev_tag)::value;
     constexpr int NEWI = REV ? 0 : NKL - 1;
-    auto seq = [&](int it) { return REV ? blk0 + SB - 1 - it : blk0 + it; };
+    auto seq = [&](int it) { return REV ? blk0 + TOT - 1 - it : blk0 + it; };
+    // first query of the run that block `blk` belongs to
+    auto run_q = [&](int blk) { return MULTI ? (blk & ~(SB - 1)) * TILE_Q : blk0 * TILE_Q; };
     auto request = [&](Stage &sg, int blk) {
         const int q0 = blk * TILE_Q;
         load_block(Qb, q0, sg.q, nt_q);
@@ -319,8 +331,9 @@ attn_tile_kernel(TileParams p) {
     // Everything the strip's first block needs is requested before anything is consumed, in
     // the order of use (loads return in order): one memory round trip for the prologue.
     u32x4_t far_k[NLD], far_v[NLD];
-    load_far(Kb, far_k);
-    load_far(Vb, far_v);
+    load_far(Kb, run_q(seq(0)), far_k);
+    load_far(Vb, run_q(seq(0)), far_v);
+    far_biases(run_q(seq(0)));
     u32x4_t halo_k[NKL][NLD], halo_v[NKL][NLD];
 #pragma unroll
     for (int c = 0; c < NKL; ++c) {
@@ -334,14 +347,15 @@ attn_tile_kernel(TileParams p) {
 
     u32x4_t Ku[KS];
     u32x2_t Vu[NJ];
-    {
+    auto far_operands = [&]() {
         u32x4_t vop[KS];
         lds_put(0, far_k);
         lds_put(1, far_v);
         lds_get(0, Ku);
         lds_get(1, vop);
         transpose_v(vop, Vu);
-    }
+    };
+    far_operands();
     u32x4_t Kl[NKL][KS];
     u32x2_t Vl[NKL][NJ];
 #pragma unroll
@@ -355,7 +369,9 @@ attn_tile_kernel(TileParams p) {
         transpose_v(vop, Vl[c]);
     }
 
-    auto process = [&](Stage &sg, int blk, Stage &nsg, int next_blk) {
+    // always_tag: `next_blk` exists, its request is unconditional.  (In a ring of stages a request
+    // under a run-time condition keeps the stage's previous contents alive as the other arm.)
+    auto process = [&](Stage &sg, int blk, Stage &nsg, int next_blk, auto always_tag) {
         const int q0 = blk * TILE_Q;
         // rows -> MFMA operand pieces
         u32x4_t Qf[KS], Vn[KS], Kt[KS], Vtn[KS];
@@ -365,7 +381,7 @@ attn_tile_kernel(TileParams p) {
         lds_put(3, sg.kt);
         lds_put(4, sg.vt);
         // this block's raw registers are consumed: request a later block's
-        if (next_blk >= 0) request(nsg, next_blk);
+        if (decltype(always_tag)::value || next_blk >= 0) request(nsg, next_blk);
         lds_get(0, Qf);
         lds_get(1, Kl[NEWI]);
         lds_get(2, Vn);
@@ -535,10 +551,28 @@ attn_tile_kernel(TileParams p) {
         }
     };
 
+    if constexpr (!MULTI) {
 #pragma unroll
-    for (int it = 0; it < SB; ++it) {
-        if (it + AHEAD < SB) process(st[it], seq(it), st[it + AHEAD], seq(it + AHEAD));
-        else process(st[it], seq(it), st[it], -1);
+        for (int it = 0; it < SB; ++it) {
+            if (it + AHEAD < SB) process(st[it], seq(it), st[it + AHEAD], seq(it + AHEAD), std::false_type{});
+            else process(st[it], seq(it), st[it], -1, std::false_type{});
+        }
+    } else {
+        // the stages are a ring that runs on across the runs; straight-line code like the single run
+#pragma unroll
+        for (int i = 0; i < TOT; ++i) {
+            const int it = i % SB, r = i / SB;
+            if (it == 0 && r > 0) {
+                far_operands();
+                far_biases(run_q(seq(i)));
+            }
+            if (it == SB - 2 && r + 1 < RUNS) {  // the next run's far block, two blocks ahead
+                load_far(Kb, run_q(seq(SB * (r + 1))), far_k);
+                load_far(Vb, run_q(seq(SB * (r + 1))), far_v);
+            }
+            if (i + AHEAD < TOT) process(st[it], seq(i), st[(it + AHEAD) % SB], seq(i + AHEAD), std::true_type{});
+            else process(st[it], seq(i), st[it], -1, std::false_type{});
+        }
     }
     };  // run
 

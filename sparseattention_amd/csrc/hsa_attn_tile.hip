@@ -20,7 +20,7 @@ constexpr int TILE_MAX_NBW_WIDE = 4;
 struct TileKnobs {
     std::atomic<int> sb{0}, wpb{0}, swizzle{1}, alternate{1};
     TileKnobs() {
-        if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4) sb = x; }
+        if (const char *e = getenv("HSA_ATTN_TILE_SB")) { int x = atoi(e); if (x == 1 || x == 2 || x == 4 || x == 8) sb = x; }
         if (const char *e = getenv("HSA_ATTN_TILE_SWZ")) swizzle = atoi(e) != 0;
         if (const char *e = getenv("HSA_ATTN_TILE_ALT")) alternate = atoi(e) != 0;
         if (const char *e = getenv("HSA_ATTN_TILE_WPB")) { int x = atoi(e); if (x >= 1 && x <= 8) wpb = x; }
@@ -33,12 +33,13 @@ static TileKnobs &tile_knobs() {
 
 // the two knobs the fp32 tile launch shares
 void attn_tile_knobs_sb_swizzle(int *sb, int *swizzle) {
-    *sb = tile_knobs().sb;
+    *sb = tile_knobs().sb > 4 ? 4 : (int)tile_knobs().sb;  // strips of more than four blocks: 16-bit kernels only
     *swizzle = tile_knobs().swizzle;
 }
 
 int attn_tile_tune(int sb, int wpb, int swizzle, int alternate) {
-    if (!(sb == -1 || sb == 0 || sb == 1 || sb == 2 || sb == 4)) return fail(HSA_ERR_INVALID, "strip length %d", sb);
+    if (!(sb == -1 || sb == 0 || sb == 1 || sb == 2 || sb == 4 || sb == 8))
+        return fail(HSA_ERR_INVALID, "strip length %d", sb);
     if (!(wpb == -1 || (wpb >= 0 && wpb <= 8))) return fail(HSA_ERR_INVALID, "wavefronts per workgroup %d", wpb);
     TileKnobs &k = tile_knobs();
     if (sb >= 0) k.sb = sb;
@@ -85,13 +86,28 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     const long block_units = (long)B * H * NB;
     const long slots = D > 64 ? 1024 : 2048;
     int sb = block_units >= 4 * slots ? 4 : (block_units >= 2 * slots ? 2 : 1);
-    if (const int forced = knobs.sb) sb = forced;
+    // long sequences: a wavefront walks two runs of four blocks, the window's neighbouring leaf
+    // blocks are then fetched once per eight blocks (B1 H16 N65536 D128 R32 302 -> 286 us,
+    // B1 H16 N16384 D128 R32 80.0 -> 73.5, B1 H16 N65536 D64 R16 156 -> 146, B8 H8 N8192 D64 79.7 ->
+    // 78.0; four runs gain nothing more at 64 channels and at 128 their code no longer fits the
+    // instruction cache: 1465 us)
+    int runs = block_units >= 16 * slots ? 2 : 1;
+    if (const int forced = knobs.sb) {
+        sb = forced > 4 ? 4 : forced;
+        runs = forced > 4 ? forced / 4 : 1;
+    }
     // four or five leaf blocks per query block: shorter strips keep the operands in registers
     if ((R + TILE_Q - 1) / TILE_Q >= (causal ? 3 : 2) && sb > 2) sb = 2;
     if ((R + TILE_Q - 1) / TILE_Q >= 4 && !knobs.sb) sb = 1;  // longer strips spill at five leaf blocks + halo
     if (!causal && (R + TILE_Q - 1) / TILE_Q > TILE_MAX_NBW) sb = 1;  // seven or nine leaf blocks: one block per wavefront
     while (sb > NB) sb >>= 1;  // NB is a power of two
-    p.NS = NB / sb;
+    // runs: strips of four blocks, one or two blocks of neighbours to either side (two: causal), no weights output
+    const int nbw_ = (R + TILE_Q - 1) / TILE_Q;
+    if (sb != 4 || weights || nbw_ < 1 || nbw_ > (causal ? 2 : 1)) runs = 1;
+    while (sb * runs > NB) runs >>= 1;
+    p.runs = runs;
+    p.NS = NB / (sb * runs);
+    sb *= runs;  // the launchers switch on the strip length
     const long units = (long)B * p.NS * H;
     if (units > 0x3fffffffL) return fail(HSA_ERR_UNSUPPORTED, "problem too large for one launch");
     p.n_units = (int)units;

@@ -21,6 +21,25 @@ static int tile_launch_one(const TileParams &p, int wpb, hipStream_t st) {
     return check_launch("attn_tile_kernel");
 }
 
+// strips of eight blocks: two runs of four (one or two blocks of neighbours, two with the causal mask)
+template <typename T, int D, int NBW, bool CAUSAL, bool LSE, int RUNS>
+static int tile_launch_runs(const TileParams &p, int wpb, hipStream_t st) {
+    if constexpr (NBW >= 1 && NBW <= (CAUSAL ? 2 : 1)) {
+        constexpr int MAXW = tile_max_wpb<D, (CAUSAL ? NBW + 1 : 2 * NBW + 1)>();
+        if (wpb > MAXW) wpb = MAXW;
+        const int nwg = (p.n_units + wpb - 1) / wpb;
+        const LaunchEvents ev = take_launch_events();
+        if (ev.start && ev.stop)
+            hipExtLaunchKernelGGL((attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, LSE, RUNS>), dim3(nwg), dim3(wpb * 64), 0,
+                                  st, ev.start, ev.stop, 0, p);
+        else
+            attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, LSE, RUNS><<<nwg, wpb * 64, 0, st>>>(p);
+        return check_launch("attn_tile_kernel (runs)");
+    } else {
+        return fail(HSA_ERR_UNSUPPORTED, "strips of more than four blocks are not built for this window radius");
+    }
+}
+
 // the variant that also writes the queries' log-sum-exp (window radius up to 16, or 32 with the
 // causal mask)
 template <typename T, int D, int NBW, bool CAUSAL>
@@ -32,6 +51,7 @@ static int tile_launch_lse(const TileParams &p, int sb, int wpb, hipStream_t st)
         case 1: attn_tile_kernel<T, D, NBW, CAUSAL, 1, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
         case 2: attn_tile_kernel<T, D, NBW, CAUSAL, 2, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
         case 4: attn_tile_kernel<T, D, NBW, CAUSAL, 4, false, true><<<nwg, wpb * 64, 0, st>>>(p); break;
+        case 8: return tile_launch_runs<T, D, NBW, CAUSAL, true, 2>(p, wpb, st);
         default: return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
     }
     return check_launch("attn_tile_kernel (log-sum-exp)");
@@ -52,6 +72,7 @@ static int tile_launch_sb(const TileParams &p, int sb, int wpb, hipStream_t st) 
         case 1: return tile_launch_one<T, D, NBW, CAUSAL, 1>(p, wpb, st);
         case 2: return tile_launch_one<T, D, NBW, CAUSAL, 2>(p, wpb, st);
         case 4: return tile_launch_one<T, D, NBW, CAUSAL, 4>(p, wpb, st);
+        case 8: return tile_launch_runs<T, D, NBW, CAUSAL, false, 2>(p, wpb, st);
     }
     return fail(HSA_ERR_UNSUPPORTED, "strip length %d not built", sb);
 }

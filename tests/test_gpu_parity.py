@@ -697,6 +697,8 @@ TILE_CASES = [  # B, N, H, D, R
     (2, 128, 4, 32, 8),
     (1, 64, 3, 32, 20),
     (1, 1024, 8, 32, 16),
+    (1, 1024, 2, 128, 32),
+    (1, 2048, 1, 64, 16),
 ]
 # window radius above 32: four or five leaf blocks per query block with the causal mask, seven or
 # nine without it
@@ -731,13 +733,17 @@ def test_attention_tile_wide_window(case, dtype, strip, tile_knobs):
 @pytest.mark.parametrize("case", TILE_CASES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("strip", [None, "1", "2", "4", "4-same-direction"])
+@pytest.mark.parametrize("strip", [None, "1", "2", "4", "4-same-direction", "8", "8-same-direction"])
 def test_attention_tile_vs_oracle(case, dtype, causal, strip, tile_knobs):
-    """Strip length forced to 1 / 2 / 4 query blocks (longer strips alternate their walking
-    direction between neighbours unless told otherwise) and the dispatcher's own choice."""
+    """Strip length forced to 1 / 2 / 4 query blocks, or to 8 (two runs of four blocks per
+    wavefront, where the window radius allows it: bit-identical to strips of four), and the
+    dispatcher's own choice.  Longer strips alternate their walking direction between neighbours
+    unless told otherwise."""
     B, N, H, D, R = case
+    alt = 1
     if strip is not None:
-        tile_knobs(int(strip[0]), -1, -1, 0 if strip.endswith("same-direction") else 1)
+        alt = 0 if strip.endswith("same-direction") else 1
+        tile_knobs(int(strip.split("-")[0]), -1, -1, alt)
     q, k, v = make_qkv(B, N, H, D, dtype, seed=N + R + D)
     t = sa.build_tree_topology(N, causal, device=DEV)
     o = oracle.topology_tables(N, causal)
@@ -746,6 +752,11 @@ def test_attention_tile_vs_oracle(case, dtype, causal, strip, tile_knobs):
     want = oracle.attention_ref(q, k, v, o["forward_idx"], o["forward_mask"] if causal else None, R,
                                 compute_dtype=torch.float64)
     assert_close(out, want, dtype, "tile")
+    if strip is not None and int(strip.split("-")[0]) > 4:
+        tile_knobs(4, -1, -1, alt)
+        four = fn.attention_forward(q.to(DEV), k.to(DEV), v.to(DEV), t["forward_idx"],
+                                    t["forward_mask"] if causal else None, R, algo="tile")
+        assert torch.equal(out, four), "two runs of four blocks against strips of four"
 
 
 @pytest.mark.parametrize("case", TILE_CASES + [(1, 256, 2, 64, 48), (1, 64, 2, 32, 24), (1, 128, 2, 128, 40), (2, 512, 2, 64, 64),
@@ -1129,7 +1140,7 @@ SAVED_BWD_CASES = [(2, 64, 2, 64, 16), (1, 128, 3, 64, 5), (2, 256, 4, 32, 16), 
 @pytest.mark.parametrize("case", SAVED_BWD_CASES)
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_attention_backward_from_saved_forward_state(case, causal, dtype):
+def test_attention_backward_from_saved_forward_state(case, causal, dtype, tile_knobs):
     """The one-pass backward (hsa_attn_bwd_saved) on the forward's output and log-sum-exp
     (hsa_attn_fwd_lse): gradients against autograd through the fp64 oracle and against the
     two-pass backward, the forward's output against the plain forward (bit for bit), and the
@@ -1153,6 +1164,11 @@ def test_attention_backward_from_saved_forward_state(case, causal, dtype):
     t = sa.build_tree_topology(N, causal, device=DEV)
     plain = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"] if causal else None, R)
     assert torch.equal(out, plain)
+    # strips of eight blocks (two runs of four per wavefront, long sequences) give the same bits
+    tile_knobs(8, -1, -1, -1)
+    out8, lse8 = fn.attention_forward_lse(qd, kd, vd, R, causal)
+    tile_knobs(0, -1, -1, -1)
+    assert torch.equal(out8, out) and torch.equal(lse8, lse)
     # lse: log2 of the sum over slots of 2^(logit * log2(e) / sqrt(D)), the sibling leaf counted twice
     L = N.bit_length() - 1
     idx = torch.as_tensor(o["forward_idx"]).long()
