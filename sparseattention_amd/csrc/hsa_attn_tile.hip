@@ -86,12 +86,15 @@ int attn_tile_dispatch(const void *q, const void *k, const void *v, void *out, f
     const long block_units = (long)B * H * NB;
     const long slots = D > 64 ? 1024 : 2048;
     int sb = block_units >= 4 * slots ? 4 : (block_units >= 2 * slots ? 2 : 1);
-    // long sequences: a wavefront walks two runs of four blocks, the window's neighbouring leaf
-    // blocks are then fetched once per eight blocks (B1 H16 N65536 D128 R32 302 -> 286 us,
-    // B1 H16 N16384 D128 R32 80.0 -> 73.5, B1 H16 N65536 D64 R16 156 -> 146, B8 H8 N8192 D64 79.7 ->
-    // 78.0; four runs gain nothing more at 64 channels and at 128 their code no longer fits the
-    // instruction cache: 1465 us)
-    int runs = block_units >= 16 * slots ? 2 : 1;
+    // long sequences with the causal mask: a wavefront walks two runs of four blocks, the window's
+    // neighbouring leaf blocks are then fetched once per eight blocks.  From eight blocks per
+    // wavefront slot on (us, strips of 4 -> 8): B1 H16 N65536 D128 R32 302 -> 286, N16384 80.0 ->
+    // 73.5, N8192 42.6 -> 39.1; B8 H8 N4096 D64 R16 40.2 -> 38.2, B1 H16 N65536 D64 156 -> 146; the
+    // headline shape (four blocks per slot) 20.4 -> 23.8, so not there.  Without the mask (three
+    // leaf blocks per query block in 256 registers) it loses: B8 H8 N8192 D64 84.3 -> 89.8.  Four
+    // runs gain nothing more at 64 channels and at 128 their code no longer fits the instruction
+    // cache (1465 us).
+    int runs = (causal && block_units >= 8 * slots) ? 2 : 1;
     if (const int forced = knobs.sb) {
         sb = forced > 4 ? 4 : forced;
         runs = forced > 4 ? forced / 4 : 1;
