@@ -1,9 +1,10 @@
 // Span attention backward in ONE pass over the strips (16-bit element types, canonical tables,
-// window radius up to 16), for callers that kept the forward's output and log-sum-exp.
+// window radius up to 16, or 32 with the causal mask), for callers that kept the forward's output
+// and log-sum-exp.
 //
 // The two-pass split (hsa_attn_bwd_tile.h) reads Q, dO and the leaf K / V twice: once per query
-// block for dQ, once per key block for dK / dV.  Here the wavefront that walks a strip of four or
-// eight query blocks also finishes dK / dV of the strip's own leaf key blocks: while a query block's
+// block for dQ, once per key block for dK / dV.  Here the wavefront that walks a strip of 4 to
+// 32 query blocks also finishes dK / dV of the strip's own leaf key blocks: while a query block's
 // operands are in registers, its contribution to each leaf key block it attends is evaluated in
 // the second orientation (S[query, key], the queries in the MFMA contraction) and added to that
 // key block's accumulators; a key block is complete once the query block after it has been done.
@@ -738,8 +739,6 @@ __global__ void __launch_bounds__(BWD_WPB * 64) attn_bwd_reduce_kernel(BwdTilePa
 template <typename T, int D>
 int attn_bwd_fused_launch_td(const BwdFusedParams &fp, bool causal, hipStream_t st);
 
-// strips of eight blocks where the sequence has that many (one neighbour's block per 128 queries
-// instead of per 64, every wavefront slot of the chip filled once at B8 H8 N2048), else of four
 // launches one variant: a workgroup is four wavefronts (heads), or the two halves of one head
 template <typename T, int D, bool CAUSAL, int SB, int NBW>
 static int bwd_fused_launch_one(const BwdFusedParams &q, hipStream_t st) {
