@@ -932,7 +932,7 @@ def test_transformer_lm_vs_oracle(activation):
 
 # ---------------------------------------------------------------- long-sequence stress (size-independent checks)
 @pytest.mark.parametrize("shape", [(1, 16, 65536, 128, 32), (1, 1, 1 << 20, 64, 16)])
-def test_long_sequence_properties(shape):
+def test_long_sequence_properties(shape, tile_knobs):
     """B1 H16 N65536 D128 bf16 R32 (the long-sequence stress shape) and a 2^20-leaf tree (20 levels,
     the far tree block nearly full): too large for the gather oracle in seconds, so check what
     the mathematics fixes plus a brute-force sample of rows."""
@@ -983,6 +983,13 @@ def test_long_sequence_properties(shape):
     # the gather kernel agrees with the tile kernel at this size
     og = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R, algo="gather")
     assert (og.float() - out.float()).abs().max() < 2e-2
+    del og
+    # at this size a wavefront walks two runs of four blocks: the same bits as strips of four, and
+    # as strips of eight forced (whatever the automatic choice is)
+    for strip in (4, 8):
+        tile_knobs(strip, -1, -1, -1)
+        forced = fn.attention_forward(qd, kd, vd, t["forward_idx"], t["forward_mask"], R, algo="tile")
+        assert torch.equal(forced, out), "strips of %d blocks" % strip
 
 
 # ---------------------------------------------------------------- backward passes
