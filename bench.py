@@ -252,7 +252,42 @@ def lm_forward_measure(steps, warmup):
            "hip_graph_replay_ms_per_forward": graph_ms,
            "calls_cross_update_Y": len(spans["cross_update_Y"]),
            "calls_hierarchical_attention": len(spans["hierarchical_attention"])}
-    del model, tok, eager, captured, graph
+    del eager, captured, graph
+    torch.cuda.empty_cache()
+    # one training step of the same model on the same batch (forward, cross-entropy on fp32 logits,
+    # backward through this library's backward kernels, SGD update): reported beside the forward,
+    # not part of `value`
+    try:
+        model.train()
+        tgt = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(1)).to(dev)
+        opt = torch.optim.SGD(model.parameters(), lr=1e-4)
+
+        def train_step():
+            opt.zero_grad(set_to_none=True)
+            logits = model(tok)
+            loss = torch.nn.functional.cross_entropy(logits.view(-1, V).float(), tgt.view(-1))
+            loss.backward()
+            opt.step()
+            return loss
+
+        for _ in range(3):
+            last = train_step()
+        torch.cuda.synchronize()
+        tr = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(4):
+                last = train_step()
+            torch.cuda.synchronize()
+            tr.append((time.perf_counter() - t0) * 1e3 / 4)
+        res["train_step_ms"] = sorted(tr)[1]
+        res["train_tokens_per_s"] = B * N / (sorted(tr)[1] * 1e-3)
+        res["train_loss_is_finite"] = bool(torch.isfinite(last).item())
+        res["train_peak_memory_GB"] = torch.cuda.max_memory_allocated() / 1e9
+        del opt, tgt, last
+    except Exception as exc:  # the forward figures stand on their own
+        res["train_step_error"] = repr(exc)[:200]
+    del model, tok
     torch.cuda.empty_cache()
     return res
 
