@@ -49,6 +49,8 @@ def parse():
     ap.add_argument("--streams", type=int, default=2,
                     help="HIP streams the steps alternate between (each step is an independent batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-train-step", action="store_true",
+                    help="cfg4: leave out the training step measured beside the forward (kernel profiles of the forward)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the brief measurements of the other configurations (detail.configs)")
@@ -154,7 +156,7 @@ LIB_LAUNCHERS = ("hsa_attn_fwd", "hsa_build_parents_fwd", "hsa_build_parents_str
                  "hsa_build_tree_fwd", "hsa_span_input_y", "hsa_topology_device", "hsa_cross_update_pack_weights")
 
 
-def lm_forward_measure(steps, warmup):
+def lm_forward_measure(steps, warmup, train_step=True):
     """cfg4: forward of the 6-layer decoder LM (d_model 512, 8 heads, FFN 2048 GELU, vocab 50257,
     bf16, B=8, N=4096, window 16, random weights, token ids uniform over the vocabulary).  Returns
     the forward time, the share of the two module calls (event pairs around them) and the GPU time
@@ -258,6 +260,8 @@ def lm_forward_measure(steps, warmup):
     # backward through this library's backward kernels, SGD update): reported beside the forward,
     # not part of `value`
     try:
+        if not train_step:
+            raise StopIteration
         model.train()
         tgt = torch.randint(0, V, (B, N), generator=torch.Generator().manual_seed(1)).to(dev)
         opt = torch.optim.SGD(model.parameters(), lr=1e-4)
@@ -285,6 +289,8 @@ def lm_forward_measure(steps, warmup):
         res["train_loss_is_finite"] = bool(torch.isfinite(last).item())
         res["train_peak_memory_GB"] = torch.cuda.max_memory_allocated() / 1e9
         del opt, tgt, last
+    except StopIteration:
+        pass
     except Exception as exc:  # the forward figures stand on their own
         res["train_step_error"] = repr(exc)[:200]
     del model, tok
@@ -293,7 +299,7 @@ def lm_forward_measure(steps, warmup):
 
 
 def lm_forward_bench(args):
-    r = lm_forward_measure(args.steps, args.warmup)
+    r = lm_forward_measure(args.steps, args.warmup, not args.no_train_step)
     print(json.dumps({
         "metric": "LM forward tokens/sec, 6L d512 h8 ffn2048 GELU vocab50257 bf16 B8 N4096 SWA16",
         "value": r["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": r["steps"], "warmup": r["warmup"],
@@ -748,7 +754,7 @@ def main():
             "cfg5": brief_config(torch, _lib, lib, hip, "cfg5", True, min(kb, 20), cs),
         }
         # the decoder LM (its own metric: tokens/s of the forward; see --workload cfg4)
-        result["detail"]["configs"]["cfg4"] = lm_forward_measure(20, 10)
+        result["detail"]["configs"]["cfg4"] = lm_forward_measure(20, 10, not args.no_train_step)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(B, H, N, D, R, causal, scale, args.cpu_seconds)
     if args.attention_only:
